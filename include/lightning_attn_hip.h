@@ -1,0 +1,99 @@
+/*
+ * C ABI of liblightning_attn_hip.so -- hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * The reference (OpenNLPLab/lightning-attention) has no native ABI: its device
+ * code is Triton-JIT launched from torch.autograd.Function bodies.  Each entry
+ * point below replaces one of those launch sites; the citation names the
+ * reference lines whose work it does.  The Python package binds these symbols
+ * with ctypes (lightning_attn/ops/hip/_lib.py).
+ *
+ * Conventions
+ *   - all pointers are device pointers owned by the caller (row-major,
+ *     contiguous unless a stride argument says otherwise);
+ *   - every call only enqueues work on `stream` (a hipStream_t passed as
+ *     void*; NULL = the default stream): no allocation, no host sync;
+ *   - the return value is 0 on success, a negative LA_E_* code for argument
+ *     errors detected on the host before anything is launched, or a positive
+ *     hipError_t reported by the launch.  la_error_string() names either;
+ *   - dtype: LA_BF16 = 0, LA_FP16 = 1, LA_FP32 = 2 (element type of q,k,v,o and
+ *     of the gradients; x,y,dy,dx for the norm).  Slopes, rstd and every
+ *     accumulator are float32;
+ *   - calls are re-entrant and thread-safe: the library keeps no mutable state.
+ */
+#ifndef LIGHTNING_ATTN_HIP_H
+#define LIGHTNING_ATTN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { LA_BF16 = 0, LA_FP16 = 1, LA_FP32 = 2 };
+
+enum {
+    LA_OK = 0,
+    LA_E_NULLPTR = -1,     /* a required pointer is NULL                      */
+    LA_E_SHAPE = -2,       /* a dimension is <= 0 or exceeds the index range  */
+    LA_E_UNSUPPORTED = -3, /* head dims / dtype outside la_supported()        */
+    LA_E_WORKSPACE = -4,   /* workspace smaller than la_workspace_bytes()     */
+    LA_E_ALIGN = -5        /* a pointer or stride is not 16-byte aligned      */
+};
+
+/* Host-only helpers (usable without a GPU). */
+const char *la_version(void);
+const char *la_error_string(int code);
+/* 1 when the attention kernels accept head dims (d, e) at this dtype:
+ * d and e multiples of 8, 8 <= d,e <= 256.  Replaces the dimension gate
+ * lightning_attn/ops/lightning_attn_interface.py:8-9,26 (is_support). */
+int la_supported(int64_t d, int64_t e, int dtype);
+/* Bytes of device scratch la_fwd (which=0) / la_bwd (which=1) need for these
+ * shapes (0 when the single-sweep path is used). */
+size_t la_workspace_bytes(int which, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype);
+
+/*
+ * Forward of decayed causal linear attention, O = (Q K^T * M_h) V with
+ * M_h[i][j] = exp(-s[h] (i-j)) for i >= j, else 0.   s == NULL means no decay
+ * (M = tril(1)).  q,k: (b,h,n,d); v,o: (b,h,n,e); s: h floats.
+ * Replaces LightningAttention2.forward + _fwd_kernel
+ * (lightning_attn/ops/triton/lightning_attn2.py:8-85, 400-434) and the no-decay
+ * twin (lightning_attn/ops/triton/lightning_attn2_no_decay.py:8-77, 369-401).
+ */
+int la_fwd(const void *q, const void *k, const void *v, const float *s, void *o,
+           int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
+           void *workspace, size_t ws_bytes, void *stream);
+
+/*
+ * Backward of the same operator: given dO (b,h,n,e) writes dq,dk (b,h,n,d) and
+ * dv (b,h,n,e), each exactly once (no read-modify-write of the gradients).
+ * Replaces LightningAttention2.backward + _bwd_intra_kernel + _bwd_inter_kernel
+ * (lightning_attn/ops/triton/lightning_attn2.py:88-395, 437-504) and the
+ * no-decay twin (lightning_attn2_no_decay.py:80-364, 404-468).
+ */
+int la_bwd(const void *q, const void *k, const void *v, const float *s, const void *dout,
+           void *dq, void *dk, void *dv,
+           int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
+           void *workspace, size_t ws_bytes, void *stream);
+
+/*
+ * SimpleRMSNorm forward: rstd[r] = 1/sqrt(mean(x[r,:]^2) + eps), y = x * rstd.
+ * x,y: rows x cols with `row_stride` elements between rows; rstd: rows floats.
+ * Replaces _SrmsNorm.forward + srms_norm_fw
+ * (lightning_attn/ops/triton/srmsnorm.py:12-33, 78-122).
+ */
+int srmsnorm_fwd(const void *x, void *y, float *rstd, int64_t rows, int64_t cols, int64_t row_stride,
+                 float eps, int dtype, void *stream);
+
+/*
+ * SimpleRMSNorm backward: xhat = x*rstd; dx = (dy - xhat*mean(xhat*dy)) * rstd.
+ * Replaces _SrmsNorm.backward + srms_norm_bwd_dx_fused
+ * (lightning_attn/ops/triton/srmsnorm.py:38-74, 125-175).
+ */
+int srmsnorm_bwd(const void *x, const void *dy, const float *rstd, void *dx,
+                 int64_t rows, int64_t cols, int64_t row_stride, int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LIGHTNING_ATTN_HIP_H */

@@ -1,0 +1,249 @@
+// SimpleRMSNorm forward / backward row kernels for gfx950.
+//
+// One 64-lane wavefront owns one row: the row is read once with 16-byte loads
+// straight into registers, reduced with cross-lane shuffles (no LDS, no
+// barrier), and written once.  Four rows per 256-thread workgroup.
+// Replaces srms_norm_fw / srms_norm_bwd_dx_fused
+// (lightning_attn/ops/triton/srmsnorm.py:12-33, 38-74).
+#include "la_common.h"
+#include "lightning_attn_hip.h"
+
+namespace la {
+
+typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
+
+template <typename T>
+struct alignas(16) Pack16 {
+    static constexpr int N = 16 / sizeof(T);
+    T v[N];
+};
+
+template <typename T>
+__device__ __forceinline__ Pack16<T> load16(const T* p) {
+    Pack16<T> r;
+    *reinterpret_cast<u32x4*>(&r) = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return r;
+}
+template <typename T>
+__device__ __forceinline__ void store16(T* p, const Pack16<T>& r) {
+    __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(&r), reinterpret_cast<u32x4*>(p));
+}
+
+// ---- register-resident rows: cols <= 64 * (16/sizeof T) * NV ---------------
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void srms_fwd_vec(const T* __restrict__ x, T* __restrict__ y,
+                                                    float* __restrict__ rstd, int64_t rows, int cols,
+                                                    int64_t stride, float eps) {
+    constexpr int E = Pack16<T>::N;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const T* xr = x + row * stride;
+    T* yr = y + row * stride;
+    Pack16<T> buf[NV];
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int c = (u * 64 + lane) * E;
+        if (c < cols) buf[u] = load16(xr + c);
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int c = (u * 64 + lane) * E;
+        if (c < cols) {
+#pragma unroll
+            for (int t = 0; t < E; ++t) {
+                const float f = (float)buf[u].v[t];
+                ss += f * f;
+            }
+        }
+    }
+    ss = wave_sum(ss);
+    const float rs = 1.0f / sqrtf(ss / (float)cols + eps);
+    if (lane == 0) rstd[row] = rs;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int c = (u * 64 + lane) * E;
+        if (c < cols) {
+            Pack16<T> o;
+#pragma unroll
+            for (int t = 0; t < E; ++t) o.v[t] = (T)((float)buf[u].v[t] * rs);
+            store16(yr + c, o);
+        }
+    }
+}
+
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void srms_bwd_vec(const T* __restrict__ x, const T* __restrict__ dy,
+                                                    const float* __restrict__ rstd, T* __restrict__ dx,
+                                                    int64_t rows, int cols, int64_t stride) {
+    constexpr int E = Pack16<T>::N;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const T* xr = x + row * stride;
+    const T* gr = dy + row * (int64_t)cols;  // dy and dx are dense (rows, cols)
+    T* dr = dx + row * (int64_t)cols;
+    Pack16<T> bx[NV], bg[NV];
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int c = (u * 64 + lane) * E;
+        if (c < cols) {
+            bx[u] = load16(xr + c);
+            bg[u] = load16(gr + c);
+        }
+    }
+    const float rs = rstd[row];
+    float acc = 0.f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int c = (u * 64 + lane) * E;
+        if (c < cols) {
+#pragma unroll
+            for (int t = 0; t < E; ++t) acc += ((float)bx[u].v[t] * rs) * (float)bg[u].v[t];
+        }
+    }
+    acc = wave_sum(acc);
+    const float m = acc / (float)cols;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int c = (u * 64 + lane) * E;
+        if (c < cols) {
+            Pack16<T> o;
+#pragma unroll
+            for (int t = 0; t < E; ++t) {
+                const float xh = (float)bx[u].v[t] * rs;
+                o.v[t] = (T)(((float)bg[u].v[t] - xh * m) * rs);
+            }
+            store16(dr + c, o);
+        }
+    }
+}
+
+// ---- any cols / any alignment: one workgroup per row, scalar accesses ------
+__device__ __forceinline__ float block_sum_256(float v, float* red) {
+    v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    const float t = red[0] + red[1] + red[2] + red[3];
+    __syncthreads();
+    return t;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void srms_fwd_any(const T* __restrict__ x, T* __restrict__ y,
+                                                    float* __restrict__ rstd, int64_t rows, int64_t cols,
+                                                    int64_t stride, float eps) {
+    __shared__ float red[4];
+    const int64_t row = blockIdx.x;
+    const T* xr = x + row * stride;
+    T* yr = y + row * stride;
+    float ss = 0.f;
+    for (int64_t c = threadIdx.x; c < cols; c += 256) {
+        const float f = (float)xr[c];
+        ss += f * f;
+    }
+    ss = block_sum_256(ss, red);
+    const float rs = 1.0f / sqrtf(ss / (float)cols + eps);
+    if (threadIdx.x == 0) rstd[row] = rs;
+    for (int64_t c = threadIdx.x; c < cols; c += 256) yr[c] = (T)((float)xr[c] * rs);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void srms_bwd_any(const T* __restrict__ x, const T* __restrict__ dy,
+                                                    const float* __restrict__ rstd, T* __restrict__ dx,
+                                                    int64_t rows, int64_t cols, int64_t stride) {
+    __shared__ float red[4];
+    const int64_t row = blockIdx.x;
+    const T* xr = x + row * stride;
+    const T* gr = dy + row * cols;
+    T* dr = dx + row * cols;
+    const float rs = rstd[row];
+    float acc = 0.f;
+    for (int64_t c = threadIdx.x; c < cols; c += 256) acc += ((float)xr[c] * rs) * (float)gr[c];
+    acc = block_sum_256(acc, red);
+    const float m = acc / (float)cols;
+    for (int64_t c = threadIdx.x; c < cols; c += 256) {
+        const float xh = (float)xr[c] * rs;
+        dr[c] = (T)(((float)gr[c] - xh * m) * rs);
+    }
+}
+
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <typename T>
+static int launch_fwd(const void* x, void* y, float* rstd, int64_t rows, int64_t cols, int64_t stride,
+                      float eps, hipStream_t st) {
+    constexpr int E = 16 / sizeof(T);
+    const T* xp = static_cast<const T*>(x);
+    T* yp = static_cast<T*>(y);
+    const bool vec = (cols % E == 0) && (stride % E == 0) && aligned16(x) && aligned16(y) && cols <= 64 * E * 16;
+    if (vec) {
+        const unsigned grid = (unsigned)((rows + 3) / 4);
+        const int nv = (int)((cols + 64 * E - 1) / (64 * E));
+#define LA_FWD(NV) hipLaunchKernelGGL((srms_fwd_vec<T, NV>), dim3(grid), dim3(256), 0, st, xp, yp, rstd, rows, (int)cols, stride, eps)
+        if (nv <= 1) LA_FWD(1);
+        else if (nv <= 2) LA_FWD(2);
+        else if (nv <= 4) LA_FWD(4);
+        else if (nv <= 8) LA_FWD(8);
+        else LA_FWD(16);
+#undef LA_FWD
+    } else {
+        hipLaunchKernelGGL((srms_fwd_any<T>), dim3((unsigned)rows), dim3(256), 0, st, xp, yp, rstd, rows, cols, stride, eps);
+    }
+    return (int)hipGetLastError();
+}
+
+template <typename T>
+static int launch_bwd(const void* x, const void* dy, const float* rstd, void* dx, int64_t rows, int64_t cols,
+                      int64_t stride, hipStream_t st) {
+    constexpr int E = 16 / sizeof(T);
+    const T* xp = static_cast<const T*>(x);
+    const T* gp = static_cast<const T*>(dy);
+    T* dp = static_cast<T*>(dx);
+    const bool vec = (cols % E == 0) && (stride % E == 0) && aligned16(x) && aligned16(dy) && aligned16(dx) &&
+                     cols <= 64 * E * 8;
+    if (vec) {
+        const unsigned grid = (unsigned)((rows + 3) / 4);
+        const int nv = (int)((cols + 64 * E - 1) / (64 * E));
+#define LA_BWD(NV) hipLaunchKernelGGL((srms_bwd_vec<T, NV>), dim3(grid), dim3(256), 0, st, xp, gp, rstd, dp, rows, (int)cols, stride)
+        if (nv <= 1) LA_BWD(1);
+        else if (nv <= 2) LA_BWD(2);
+        else if (nv <= 4) LA_BWD(4);
+        else LA_BWD(8);
+#undef LA_BWD
+    } else {
+        hipLaunchKernelGGL((srms_bwd_any<T>), dim3((unsigned)rows), dim3(256), 0, st, xp, gp, rstd, dp, rows, cols, stride);
+    }
+    return (int)hipGetLastError();
+}
+
+}  // namespace la
+
+extern "C" int srmsnorm_fwd(const void* x, void* y, float* rstd, int64_t rows, int64_t cols, int64_t row_stride,
+                            float eps, int dtype, void* stream) {
+    if (!x || !y || !rstd) return LA_E_NULLPTR;
+    if (rows < 0 || cols <= 0 || row_stride < cols || rows > 0x7fffffffLL) return LA_E_SHAPE;
+    if (rows == 0) return LA_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case LA_BF16: return la::launch_fwd<__bf16>(x, y, rstd, rows, cols, row_stride, eps, st);
+        case LA_FP16: return la::launch_fwd<_Float16>(x, y, rstd, rows, cols, row_stride, eps, st);
+        case LA_FP32: return la::launch_fwd<float>(x, y, rstd, rows, cols, row_stride, eps, st);
+        default: return LA_E_UNSUPPORTED;
+    }
+}
+
+extern "C" int srmsnorm_bwd(const void* x, const void* dy, const float* rstd, void* dx, int64_t rows, int64_t cols,
+                            int64_t row_stride, int dtype, void* stream) {
+    if (!x || !dy || !rstd || !dx) return LA_E_NULLPTR;
+    if (rows < 0 || cols <= 0 || row_stride < cols || rows > 0x7fffffffLL) return LA_E_SHAPE;
+    if (rows == 0) return LA_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case LA_BF16: return la::launch_bwd<__bf16>(x, dy, rstd, dx, rows, cols, row_stride, st);
+        case LA_FP16: return la::launch_bwd<_Float16>(x, dy, rstd, dx, rows, cols, row_stride, st);
+        case LA_FP32: return la::launch_bwd<float>(x, dy, rstd, dx, rows, cols, row_stride, st);
+        default: return LA_E_UNSUPPORTED;
+    }
+}

@@ -1,0 +1,49 @@
+"""Public dispatch function, lightning_attn/ops/lightning_attn_interface.py:16-65.
+
+The reference pads e to a power of two and splits d > 128 into <= 64-wide
+slices because its Triton tiles need that; the HIP kernels tile any multiple of
+8 up to 256 natively, so neither happens here.  Feature dims above 256 are
+split into 256-wide slices of q/k whose partial outputs add up (the scores are
+additive over feature slices)."""
+from .hip import _lib
+from .hip.lightning_attn2 import lightning_attn2, lightning_attn2_no_decay
+
+_VARIANTS = ("chunk_loop", "parallel")
+_MAX_DIM = 256
+
+
+def is_support(dim):
+    """True when a feature dim is usable: a positive multiple of 8."""
+    return dim > 0 and dim % 8 == 0
+
+
+def lightning_attn_func(q, k, v, s=None, variant="chunk_loop"):
+    """o = (q k^T * M) v with M[i,j] = exp(-s_h (i-j)) [i >= j]; s=None means no decay.
+
+    q, k: (b, h, n, d); v: (b, h, n, e); s: h float32 rates (any shape with h
+    elements) or None.  Returns (b, h, n, e) in q.dtype; differentiable in
+    q, k, v."""
+    if variant not in _VARIANTS:
+        raise ValueError("variant must be one of %s, got %r" % (_VARIANTS, variant))
+    b, h, n, d = q.shape
+    e = v.shape[-1]
+    assert is_support(d) and is_support(e), "feature dims must be multiples of 8 (got d=%d, e=%d)" % (d, e)
+
+    def run(q1, k1, v1):
+        if s is None:
+            return lightning_attn2_no_decay(q1, k1, v1)
+        return lightning_attn2(q1, k1, v1, s)
+
+    if e > _MAX_DIM:
+        # output columns are independent: cut v
+        outs = [lightning_attn_func(q, k, v[..., c : c + _MAX_DIM], s, variant) for c in range(0, e, _MAX_DIM)]
+        import torch
+
+        return torch.cat(outs, dim=-1)
+    if d > _MAX_DIM:
+        o = None
+        for c in range(0, d, _MAX_DIM):
+            part = run(q[..., c : c + _MAX_DIM], k[..., c : c + _MAX_DIM], v)
+            o = part if o is None else o + part
+        return o
+    return run(q, k, v)
