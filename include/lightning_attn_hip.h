@@ -45,7 +45,7 @@ enum {
 const char *la_version(void);
 const char *la_error_string(int code);
 /* 1 when the attention kernels accept head dims (d, e) at this dtype:
- * d and e multiples of 8, 8 <= d,e <= 256.  Replaces the dimension gate
+ * d and e multiples of 8, 8 <= d,e <= 256 (<= 128 for float32).  Replaces the dimension gate
  * lightning_attn/ops/lightning_attn_interface.py:8-9,26 (is_support). */
 int la_supported(int64_t d, int64_t e, int dtype);
 /* Bytes of device scratch la_fwd (which=0) / la_bwd (which=1) need for these

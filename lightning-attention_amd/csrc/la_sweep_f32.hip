@@ -1,0 +1,258 @@
+// float32 variant of the sweep (see la_sweep.hip for the algorithm): the same
+// block recurrence and work split, with every product on the fp32 matrix
+// instruction v_mfma_f32_16x16x4_f32 (one A and one B element per lane:
+// row/column = lane % 16, contraction slot = lane / 16).  Nothing is rounded
+// below float32, so the result is within float32 accumulation error of the
+// exact value.  This is the accuracy path, not the throughput path.
+#include "la_common.h"
+#include "lightning_attn_hip.h"
+
+namespace la {
+
+struct SweepArgsF32 {
+    const float* x;
+    const float* y;
+    const float* z;
+    float* out;
+    const float* s;
+    int64_t n;
+    int dk, dv, h, bh, nslice;
+};
+
+__device__ __forceinline__ f32x4 mma4(float a, float b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+template <int DKP, bool REVERSE, bool DECAY>
+__global__ __launch_bounds__(256, 1) void la_sweep_f32_kernel(SweepArgsF32 a) {
+    constexpr int XS = DKP + 4;   // row stride (floats) of the x / y tiles
+    constexpr int ZS = 64 + 4;    // row stride of the z slice and the P tile
+    constexpr int KT = DKP / 16;  // 16-row state tiles
+    constexpr int XC = DKP / 16;  // 16-byte chunks per thread for an x / y tile
+    extern __shared__ __align__(16) unsigned char smem[];
+    float* Xs = reinterpret_cast<float*>(smem);
+    float* Ys = Xs + 64 * XS;
+    float* Zs = Ys + 64 * XS;
+    float* Ps = Zs + 64 * ZS;
+
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int unit = xcd + 8 * (local / a.nslice);
+    const int slice = local % a.nslice;
+    if (unit >= a.bh) return;
+
+    const int tid = threadIdx.x;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63, r = lane & 15, g = lane >> 4;
+    const int64_t n = a.n;
+    const int dk = a.dk, dv = a.dv;
+    const float* xg = a.x + (int64_t)unit * n * dk;
+    const float* yg = a.y + (int64_t)unit * n * dk;
+    const float* zg = a.z + (int64_t)unit * n * dv;
+    float* og = a.out + (int64_t)unit * n * dv;
+    const int col0 = slice * 64;
+    const bool wave_active = (col0 + 16 * w) < dv;
+
+    float rate = 0.f;
+    if (DECAY) rate = a.s[unit % a.h];
+
+    float dfac[4][4], ofac[4], zfac[4][4], lamB = 1.f;
+#pragma unroll
+    for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int i = 16 * w + r, j = 16 * jt + 4 * g + v;
+            const int diff = REVERSE ? (j - i) : (i - j);
+            dfac[jt][v] = diff >= 0 ? (DECAY ? expf(-rate * (float)diff) : 1.f) : 0.f;
+            zfac[jt][v] = DECAY ? expf(-rate * (float)(REVERSE ? j : 64 - j)) : 1.f;
+        }
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int i = 16 * it + r;
+        ofac[it] = DECAY ? expf(-rate * (float)(REVERSE ? 64 - i : i)) : 1.f;
+    }
+    if (DECAY) lamB = expf(-rate * 64.f);
+
+    f32x4 st[KT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) st[kt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    const int64_t nblk = (n + 63) / 64;
+    uint4 xr[XC], yr[XC], zr[4];
+
+    auto load_block = [&](int64_t t) {
+        const int64_t tok0 = t * 64;
+#pragma unroll
+        for (int u = 0; u < XC; ++u) {
+            const int c = tid + 256 * u;
+            const int row = c / (DKP / 4), col = (c % (DKP / 4)) * 4;
+            const bool ok = (tok0 + row < n) && (col < dk);
+            xr[u] = ok ? *reinterpret_cast<const uint4*>(xg + (tok0 + row) * dk + col) : make_uint4(0, 0, 0, 0);
+            yr[u] = ok ? *reinterpret_cast<const uint4*>(yg + (tok0 + row) * dk + col) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int c = tid + 256 * u;
+            const int row = c / 16, col = (c % 16) * 4;
+            const bool ok = (tok0 + row < n) && (col0 + col < dv);
+            zr[u] = ok ? *reinterpret_cast<const uint4*>(zg + (tok0 + row) * dv + col0 + col) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto stage_block = [&]() {
+#pragma unroll
+        for (int u = 0; u < XC; ++u) {
+            const int c = tid + 256 * u;
+            const int row = c / (DKP / 4), col = (c % (DKP / 4)) * 4;
+            *reinterpret_cast<uint4*>(Xs + row * XS + col) = xr[u];
+            *reinterpret_cast<uint4*>(Ys + row * XS + col) = yr[u];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int c = tid + 256 * u;
+            const int row = c / 16, col = (c % 16) * 4;
+            *reinterpret_cast<uint4*>(Zs + row * ZS + col) = zr[u];
+        }
+    };
+
+    for (int c = tid; c < 64 * ZS / 4; c += 256) reinterpret_cast<uint4*>(Ps)[c] = make_uint4(0, 0, 0, 0);
+    load_block(REVERSE ? nblk - 1 : 0);
+    stage_block();
+    __syncthreads();
+
+    const int jlo = REVERSE ? w : 0, jhi = REVERSE ? 3 : w;
+
+    for (int64_t it = 0; it < nblk; ++it) {
+        const int64_t t = REVERSE ? nblk - 1 - it : it;
+        const bool have_next = it + 1 < nblk;
+        if (have_next) load_block(REVERSE ? t - 1 : t + 1);
+
+        // 1. S^T tiles (rows j, columns i in [16w, 16w+16)) -> masked, decayed P[i][j]
+        {
+            f32x4 sacc[4];
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) sacc[jt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+            for (int k0 = 0; k0 < DKP; k0 += 4) {
+                const float bx = Xs[(16 * w + r) * XS + k0 + g];
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) {
+                    if (jt >= jlo && jt <= jhi) sacc[jt] = mma4(Ys[(16 * jt + r) * XS + k0 + g], bx, sacc[jt]);
+                }
+            }
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) {
+                if (jt >= jlo && jt <= jhi) {
+                    f32x4 p;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) p[v] = sacc[jt][v] * dfac[jt][v];
+                    *reinterpret_cast<f32x4*>(Ps + (16 * w + r) * ZS + 16 * jt + 4 * g) = p;
+                }
+            }
+        }
+        __syncthreads();
+
+        if (wave_active) {
+            // z[j][16w + r] for the 16 tokens j = 16jt + 4g + v this lane contracts over
+            float zf[4][4];
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) zf[jt][v] = Zs[(16 * jt + 4 * g + v) * ZS + 16 * w + r];
+
+            f32x4 oacc[4];
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+                oacc[i4] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                // 2a. inter-block: contraction slot g of step (kt, v) is feature 16kt + 4g + v
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+                    const f32x4 bx = *reinterpret_cast<const f32x4*>(Xs + (16 * i4 + r) * XS + 16 * kt + 4 * g);
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) oacc[i4] = mma4(st[kt][v], bx[v], oacc[i4]);
+                }
+                if (DECAY) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) oacc[i4][v] *= ofac[i4];
+                }
+                // 2b. intra-block: slot g of step (jt, v) is token 16jt + 4g + v
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) {
+                    const bool need = REVERSE ? (jt >= i4) : (jt <= i4);
+                    if (need) {
+                        const f32x4 bp = *reinterpret_cast<const f32x4*>(Ps + (16 * i4 + r) * ZS + 16 * jt + 4 * g);
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) oacc[i4] = mma4(zf[jt][v], bp[v], oacc[i4]);
+                    }
+                }
+            }
+            const int col = col0 + 16 * w + 4 * g;
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+                const int64_t tok = t * 64 + 16 * i4 + r;
+                if (tok < n && col < dv) *reinterpret_cast<f32x4*>(og + tok * dv + col) = oacc[i4];
+            }
+            // 3. state = lam^64 state + y^T (z * Lupd)
+            if (have_next) {
+                if (DECAY) {
+#pragma unroll
+                    for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) zf[jt][v] *= zfac[jt][v];
+#pragma unroll
+                    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) st[kt][v] *= lamB;
+                }
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+                    for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+                        for (int v = 0; v < 4; ++v)
+                            st[kt] = mma4(Ys[(16 * jt + 4 * g + v) * XS + 16 * kt + r], zf[jt][v], st[kt]);
+                }
+            }
+        }
+        __syncthreads();
+        if (have_next) {
+            stage_block();
+            __syncthreads();
+        }
+    }
+}
+
+template <int DKP, bool REVERSE, bool DECAY>
+static int launch_one_f32(const SweepArgsF32& a, hipStream_t st) {
+    constexpr size_t lds = (size_t)(2 * 64 * (DKP + 4) + 2 * 64 * 68) * sizeof(float);
+    auto kern = la_sweep_f32_kernel<DKP, REVERSE, DECAY>;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+    }
+    const int units8 = (a.bh + 7) / 8 * 8;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(units8 * a.nslice)), dim3(256), lds, st, a);
+    return (int)hipGetLastError();
+}
+
+template <bool REVERSE>
+static int launch_dir_f32(const SweepArgsF32& a, hipStream_t st) {
+    const bool decay = a.s != nullptr;
+#define LA_GO(DKP) (decay ? launch_one_f32<DKP, REVERSE, true>(a, st) : launch_one_f32<DKP, REVERSE, false>(a, st))
+    if (a.dk <= 32) return LA_GO(32);
+    if (a.dk <= 64) return LA_GO(64);
+    return LA_GO(128);
+#undef LA_GO
+}
+
+int sweep_f32(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
+              int64_t n, int64_t dk, int64_t dv, bool reverse, hipStream_t st) {
+    if (dk > 128) return LA_E_UNSUPPORTED;
+    SweepArgsF32 a;
+    a.x = static_cast<const float*>(x); a.y = static_cast<const float*>(y); a.z = static_cast<const float*>(z);
+    a.out = static_cast<float*>(out); a.s = s;
+    a.n = n; a.dk = (int)dk; a.dv = (int)dv; a.h = (int)h; a.bh = (int)bh;
+    a.nslice = (int)((dv + 63) / 64);
+    return reverse ? launch_dir_f32<true>(a, st) : launch_dir_f32<false>(a, st);
+}
+
+}  // namespace la

@@ -222,9 +222,10 @@ static int launch_bwd(const void* x, const void* dy, const float* rstd, void* dx
 
 extern "C" int srmsnorm_fwd(const void* x, void* y, float* rstd, int64_t rows, int64_t cols, int64_t row_stride,
                             float eps, int dtype, void* stream) {
-    if (!x || !y || !rstd) return LA_E_NULLPTR;
     if (rows < 0 || cols <= 0 || row_stride < cols || rows > 0x7fffffffLL) return LA_E_SHAPE;
-    if (rows == 0) return LA_OK;
+    if (dtype != LA_BF16 && dtype != LA_FP16 && dtype != LA_FP32) return LA_E_UNSUPPORTED;
+    if (rows == 0) return LA_OK;  // empty tensors may carry null pointers
+    if (!x || !y || !rstd) return LA_E_NULLPTR;
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (dtype) {
         case LA_BF16: return la::launch_fwd<__bf16>(x, y, rstd, rows, cols, row_stride, eps, st);
@@ -236,9 +237,10 @@ extern "C" int srmsnorm_fwd(const void* x, void* y, float* rstd, int64_t rows, i
 
 extern "C" int srmsnorm_bwd(const void* x, const void* dy, const float* rstd, void* dx, int64_t rows, int64_t cols,
                             int64_t row_stride, int dtype, void* stream) {
-    if (!x || !dy || !rstd || !dx) return LA_E_NULLPTR;
     if (rows < 0 || cols <= 0 || row_stride < cols || rows > 0x7fffffffLL) return LA_E_SHAPE;
+    if (dtype != LA_BF16 && dtype != LA_FP16 && dtype != LA_FP32) return LA_E_UNSUPPORTED;
     if (rows == 0) return LA_OK;
+    if (!x || !dy || !rstd || !dx) return LA_E_NULLPTR;
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (dtype) {
         case LA_BF16: return la::launch_bwd<__bf16>(x, dy, rstd, dx, rows, cols, row_stride, st);

@@ -2,14 +2,14 @@
 
 The reference pads e to a power of two and splits d > 128 into <= 64-wide
 slices because its Triton tiles need that; the HIP kernels tile any multiple of
-8 up to 256 natively, so neither happens here.  Feature dims above 256 are
-split into 256-wide slices of q/k whose partial outputs add up (the scores are
-additive over feature slices)."""
-from .hip import _lib
+8 up to 256 natively (128 for float32), so neither happens here.  Larger feature
+dims are split into slices of q/k whose partial outputs add up (the scores are
+additive over feature slices) and into column groups of v."""
+import torch
+
 from .hip.lightning_attn2 import lightning_attn2, lightning_attn2_no_decay
 
 _VARIANTS = ("chunk_loop", "parallel")
-_MAX_DIM = 256
 
 
 def is_support(dim):
@@ -29,6 +29,8 @@ def lightning_attn_func(q, k, v, s=None, variant="chunk_loop"):
     e = v.shape[-1]
     assert is_support(d) and is_support(e), "feature dims must be multiples of 8 (got d=%d, e=%d)" % (d, e)
 
+    _MAX_DIM = 128 if q.dtype == torch.float32 else 256
+
     def run(q1, k1, v1):
         if s is None:
             return lightning_attn2_no_decay(q1, k1, v1)
@@ -37,8 +39,6 @@ def lightning_attn_func(q, k, v, s=None, variant="chunk_loop"):
     if e > _MAX_DIM:
         # output columns are independent: cut v
         outs = [lightning_attn_func(q, k, v[..., c : c + _MAX_DIM], s, variant) for c in range(0, e, _MAX_DIM)]
-        import torch
-
         return torch.cat(outs, dim=-1)
     if d > _MAX_DIM:
         o = None

@@ -1,0 +1,83 @@
+"""Host-side behaviour that needs no GPU: the C-ABI library loads and exports
+what include/lightning_attn_hip.h declares, argument validation, error paths."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from lightning_attn.ops import SimpleRMSNorm, lightning_attn_func, lightning_attn2, lightning_attn2_no_decay
+from lightning_attn.ops.hip import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "lightning_attn_hip.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b((?:la|srmsnorm)_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_symbols()
+    assert set(names) == set(_lib.SYMBOLS), names
+    assert os.path.exists(_lib.LIB_PATH), "build the library first: python lightning-attention_amd/build.py"
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(raw, n), n
+
+
+def test_host_only_entry_points():
+    L = _lib.lib()
+    assert b"gfx950" in L.la_version()
+    for d, e, dt, want in ((128, 128, 0, 1), (192, 192, 0, 1), (16, 64, 1, 1), (8, 256, 0, 1), (128, 128, 2, 1),
+                           (4, 64, 0, 0), (100, 64, 0, 0), (264, 64, 0, 0), (64, 0, 0, 0), (64, 64, 7, 0)):
+        assert L.la_supported(d, e, dt) == want, (d, e, dt)
+    assert L.la_error_string(0) == b"success"
+    assert b"NULL" in L.la_error_string(-1)
+    assert L.la_workspace_bytes(0, 4, 32, 8192, 128, 128, 0) >= 0
+    # argument errors are reported before any launch, so they are testable without a device
+    assert L.la_fwd(None, None, None, None, None, 1, 1, 64, 64, 64, 0, None, 0, None) == -1
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.addressof(buf)
+    p16 = (p + 15) & ~15
+    assert L.la_fwd(p16, p16, p16, None, p16, 1, 1, 64, 100, 64, 0, None, 0, None) == -3
+    assert L.la_fwd(p16, p16, p16, None, p16, 1, 0, 64, 64, 64, 0, None, 0, None) == -2
+    assert L.la_fwd(p16 + 2, p16, p16, None, p16, 1, 1, 64, 64, 64, 0, None, 0, None) == -5
+    assert L.la_bwd(p16, p16, p16, None, None, p16, p16, p16, 1, 1, 64, 64, 64, 0, None, 0, None) == -1
+    assert L.srmsnorm_fwd(None, None, None, 4, 64, 64, 1e-6, 0, None) == -1
+    assert L.srmsnorm_fwd(p16, p16, p16, 4, 0, 64, 1e-6, 0, None) == -2
+    assert L.srmsnorm_fwd(p16, p16, p16, 4, 64, 32, 1e-6, 0, None) == -2
+    assert L.srmsnorm_fwd(p16, p16, p16, 4, 64, 64, 1e-6, 9, None) == -3
+    # empty problems succeed without touching the device
+    assert L.la_fwd(p16, p16, p16, None, p16, 0, 4, 64, 64, 64, 0, None, 0, None) == 0
+    assert L.srmsnorm_bwd(p16, p16, p16, p16, 0, 64, 64, 0, None) == 0
+
+
+def test_no_cpu_fallback():
+    q = torch.randn(1, 2, 16, 16)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        lightning_attn_func(q, q, q, torch.ones(2, 1, 1))
+    with pytest.raises(RuntimeError, match="HIP device"):
+        lightning_attn2_no_decay(q, q, q)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        SimpleRMSNorm(16)(q)
+    with pytest.raises(ValueError):
+        lightning_attn2(q, q, q, None)
+
+
+def test_interface_validation():
+    q = torch.randn(1, 2, 16, 12)
+    with pytest.raises(AssertionError):
+        lightning_attn_func(q, q, q)  # d = 12 is not a multiple of 8
+    with pytest.raises(ValueError):
+        lightning_attn_func(torch.randn(1, 2, 16, 16), torch.randn(1, 2, 16, 16), torch.randn(1, 2, 16, 16), None, "ring")
+
+
+def test_missing_library_is_an_error(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/liblightning_attn_hip.so")
+    with pytest.raises(RuntimeError, match="not built"):
+        _lib.lib()
