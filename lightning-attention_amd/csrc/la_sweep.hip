@@ -8,17 +8,21 @@
 //     dK = sweep_rev(V , dO, Q )      dV = sweep_rev(K , Q , dO)
 // (lightning_attn/ops/triton/lightning_attn2.py:8-85 forward, :88-395 backward.)
 //
-// The sequence is cut into blocks of 64 tokens.  A workgroup (4 wavefronts)
-// owns one (batch, head, 64-column slice of z/out) and walks the blocks in
-// order, carrying the dk x 64 slice of the state  S = sum lam^.. y_j^T z_j  in
-// fp32 MFMA accumulators.  Wavefront w owns 16 of the 64 columns:
-//     1. S^T tile  (y x^T) for its 16 tokens i        -> decay/mask -> P in LDS
-//     2. out^T[c,i] = Lout[i] * (state^T x^T) + z^T P^T    (two MFMA chains)
-//     3. state     = lam^64 * state + y^T (z * Lupd)
+// The sequence is cut into blocks of 64 tokens.  A workgroup of 8 wavefronts owns
+// one (batch, head, 64-column slice of z/out) and walks the blocks in order.  The
+// wavefronts are specialised so that every SIMD holds two waves with different
+// instruction mixes:
+//   waves 0-3 ("score" waves)   S^T = y x^T tiles -> decay/mask -> P (LDS);
+//                               out^T = inter + z^T P^T ; store out
+//   waves 4-7 ("state" waves)   own the dk x 16 column slab of the state
+//                               S = sum lam^.. y_j^T z_j in fp32 accumulators;
+//                               inter = Lout * (state^T x^T) -> LDS;
+//                               state = lam^64 state + y^T (z * Lupd)
 // State and z^T fragments never leave registers: the accumulator layout of one
-// MFMA is reused as the A operand of the next with a matching permutation of
-// the contraction index on the B side.  Transposed operands (y^T, z^T) are
-// fetched with the LDS transpose read ds_read_b64_tr_b16.
+// MFMA is reused as the A operand of the next with a matching permutation of the
+// contraction index on the B side.  Transposed operands (y^T, z^T) come from the
+// LDS transpose read ds_read_b64_tr_b16.  x/y/z tiles are double-buffered in LDS
+// (global -> registers one block ahead -> LDS), two barriers per block.
 #include "la_common.h"
 #include "lightning_attn_hip.h"
 
@@ -73,21 +77,43 @@ __device__ __forceinline__ V8 cat(V4 a, V4 b) {
     return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// The 10 non-masked 16x16 tiles of the 64x64 score block, dealt to the four score
+// waves: slot 0 is tile (jt0, itA), slots 1,2 are (jt1, itB), (jt2, itB); -1 = none.
+// Written for the forward direction (jt <= it); the reverse direction mirrors
+// both indices (3 - jt, 3 - it).
+struct TileDeal {
+    int itA, jt0, itB, jt1, jt2;
+};
+__device__ __constant__ const TileDeal kDeal[4] = {
+    {3, 0, 3, 1, 2},
+    {3, 3, 2, 0, 1},
+    {2, 2, 1, 0, 1},
+    {0, 0, -1, -1, -1},
+};
+
+template <int DKP>
+struct SweepLds {
+    static constexpr int XS = DKP + 8;  // row stride (elements) of the x / y tiles
+    static constexpr int ZS = 64 + 8;   // row stride of the z slice and the P tile
+    static constexpr int NBUF = DKP <= 192 ? 2 : 1;
+    static constexpr int TILE = 2 * 64 * XS + 64 * ZS;  // elements of one x+y+z buffer
+    static constexpr size_t bytes(size_t elt) { return (size_t)(NBUF * TILE + 64 * ZS) * elt + 4 * 4 * 64 * 16; }
+};
+
 template <typename T, int DKP, bool REVERSE, bool DECAY>
-__global__ __launch_bounds__(256, 1) void la_sweep_kernel(SweepArgs a) {
+__global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
     typedef Mma<T> M;
     typedef typename M::V8 V8;
     typedef typename M::V4 V4;
-    constexpr int XS = DKP + 8;   // row stride (elements) of the x / y tiles
-    constexpr int ZS = 64 + 8;    // row stride of the z slice and the P tile
+    typedef SweepLds<DKP> L;
+    constexpr int XS = L::XS, ZS = L::ZS, NBUF = L::NBUF;
     constexpr int KS = DKP / 32;  // 32-wide contraction steps over the feature dim
     constexpr int KT = DKP / 16;  // 16-row state tiles
-    constexpr int XC = DKP / 32;  // 16-byte chunks per thread for an x / y tile
+    constexpr int XC = DKP / 64;  // 16-byte chunks per thread for an x / y tile (512 threads)
     extern __shared__ __align__(16) unsigned char smem[];
-    T* Xs = reinterpret_cast<T*>(smem);
-    T* Ys = Xs + 64 * XS;
-    T* Zs = Ys + 64 * XS;
-    T* Ps = Zs + 64 * ZS;
+    T* tiles = reinterpret_cast<T*>(smem);
+    T* Ps = tiles + NBUF * L::TILE;
+    f32x4* Ob = reinterpret_cast<f32x4*>(Ps + 64 * ZS);  // [wave][i4][lane]
 
     // Workgroups are dealt round-robin to the 8 XCDs by linear id; keep the
     // column slices of one head on one XCD so their x / y re-reads share an L2.
@@ -97,7 +123,9 @@ __global__ __launch_bounds__(256, 1) void la_sweep_kernel(SweepArgs a) {
     if (unit >= a.bh) return;
 
     const int tid = threadIdx.x;
-    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool state_role = wave >= 4;
+    const int w = wave & 3;
     const int lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int64_t n = a.n;
     const int dk = a.dk, dv = a.dv;
@@ -106,24 +134,36 @@ __global__ __launch_bounds__(256, 1) void la_sweep_kernel(SweepArgs a) {
     const T* zg = static_cast<const T*>(a.z) + (int64_t)unit * n * dv;
     T* og = static_cast<T*>(a.out) + (int64_t)unit * n * dv;
     const int col0 = slice * 64;
-    const bool wave_active = (col0 + 16 * w) < dv;
+    const bool cols_active = (col0 + 16 * w) < dv;
 
     float rate = 0.f;
     if (DECAY) rate = a.s[unit % a.h];
 
-    // ---- per-lane decay tables (every factor <= 1) --------------------------
-    float dfac[4][4];  // mask * decay of the S^T tile: token i = 16w + r, j = 16jt + 4g + v
+    // ---- score-wave constants: its tiles and their mask * decay factors -------
+    TileDeal deal = kDeal[w];
+    if (REVERSE) {
+        deal.itA = 3 - deal.itA; deal.jt0 = 3 - deal.jt0;
+        if (deal.itB >= 0) { deal.itB = 3 - deal.itB; deal.jt1 = 3 - deal.jt1; deal.jt2 = 3 - deal.jt2; }
+    }
+    const int itA = __builtin_amdgcn_readfirstlane(deal.itA), jt0 = __builtin_amdgcn_readfirstlane(deal.jt0);
+    const int itB = __builtin_amdgcn_readfirstlane(deal.itB), jt1 = __builtin_amdgcn_readfirstlane(deal.jt1);
+    const int jt2 = __builtin_amdgcn_readfirstlane(deal.jt2);
+    float dfac[3][4];
+    {
+        const int its[3] = {itA, itB, itB}, jts[3] = {jt0, jt1, jt2};
+#pragma unroll
+        for (int sl = 0; sl < 3; ++sl)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int i = 16 * its[sl] + r, j = 16 * jts[sl] + 4 * g + v;
+                const int diff = REVERSE ? (j - i) : (i - j);
+                dfac[sl][v] = diff >= 0 ? (DECAY ? expf(-rate * (float)diff) : 1.f) : 0.f;
+            }
+    }
+    // ---- state-wave constants (every factor <= 1) ----------------------------
     float ofac[4];     // scale of the inter-block term for token i = 16it + r
     float zfac[2][8];  // scale of token j = 32ks + 8g + u in the state update
     float lamB = 1.f;
-#pragma unroll
-    for (int jt = 0; jt < 4; ++jt)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            const int i = 16 * w + r, j = 16 * jt + 4 * g + v;
-            const int diff = REVERSE ? (j - i) : (i - j);
-            dfac[jt][v] = diff >= 0 ? (DECAY ? expf(-rate * (float)diff) : 1.f) : 0.f;
-        }
     if (DECAY) {
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
@@ -145,92 +185,99 @@ __global__ __launch_bounds__(256, 1) void la_sweep_kernel(SweepArgs a) {
     for (int kt = 0; kt < KT; ++kt) st[kt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
     const int64_t nblk = (n + 63) / 64;
-    uint4 xr[XC], yr[XC], zr[2];
+    uint4 xr[XC], yr[XC], zr;
 
     auto load_block = [&](int64_t t) {
         const int64_t tok0 = t * 64;
 #pragma unroll
         for (int u = 0; u < XC; ++u) {
-            const int c = tid + 256 * u;
+            const int c = tid + 512 * u;
             const int row = c / (DKP / 8), col = (c % (DKP / 8)) * 8;
             const bool ok = (tok0 + row < n) && (col < dk);
             xr[u] = ok ? *reinterpret_cast<const uint4*>(xg + (tok0 + row) * dk + col) : make_uint4(0, 0, 0, 0);
             yr[u] = ok ? *reinterpret_cast<const uint4*>(yg + (tok0 + row) * dk + col) : make_uint4(0, 0, 0, 0);
         }
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int c = tid + 256 * u;
-            const int row = c / 8, col = (c % 8) * 8;
+        {
+            const int row = tid / 8, col = (tid % 8) * 8;
             const bool ok = (tok0 + row < n) && (col0 + col < dv);
-            zr[u] = ok ? *reinterpret_cast<const uint4*>(zg + (tok0 + row) * dv + col0 + col) : make_uint4(0, 0, 0, 0);
+            zr = ok ? *reinterpret_cast<const uint4*>(zg + (tok0 + row) * dv + col0 + col) : make_uint4(0, 0, 0, 0);
         }
     };
-    auto stage_block = [&]() {
+    auto stage_block = [&](int buf) {
+        T* Xd = tiles + buf * L::TILE;
+        T* Yd = Xd + 64 * XS;
+        T* Zd = Yd + 64 * XS;
 #pragma unroll
         for (int u = 0; u < XC; ++u) {
-            const int c = tid + 256 * u;
+            const int c = tid + 512 * u;
             const int row = c / (DKP / 8), col = (c % (DKP / 8)) * 8;
-            *reinterpret_cast<uint4*>(Xs + row * XS + col) = xr[u];
-            *reinterpret_cast<uint4*>(Ys + row * XS + col) = yr[u];
+            *reinterpret_cast<uint4*>(Xd + row * XS + col) = xr[u];
+            *reinterpret_cast<uint4*>(Yd + row * XS + col) = yr[u];
         }
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int c = tid + 256 * u;
-            const int row = c / 8, col = (c % 8) * 8;
-            *reinterpret_cast<uint4*>(Zs + row * ZS + col) = zr[u];
+        {
+            const int row = tid / 8, col = (tid % 8) * 8;
+            *reinterpret_cast<uint4*>(Zd + row * ZS + col) = zr;
         }
     };
 
     // zero P once: tiles on the masked side of the diagonal are never written
-    for (int c = tid; c < 64 * ZS / 8; c += 256) reinterpret_cast<uint4*>(Ps)[c] = make_uint4(0, 0, 0, 0);
+    for (int c = tid; c < 64 * ZS / 8; c += 512) reinterpret_cast<uint4*>(Ps)[c] = make_uint4(0, 0, 0, 0);
     load_block(REVERSE ? nblk - 1 : 0);
-    stage_block();
+    stage_block(0);
     __syncthreads();
-
-    const int jlo = REVERSE ? w : 0, jhi = REVERSE ? 3 : w;
 
     for (int64_t it = 0; it < nblk; ++it) {
         const int64_t t = REVERSE ? nblk - 1 - it : it;
         const bool have_next = it + 1 < nblk;
+        const int buf = NBUF == 2 ? (int)(it & 1) : 0;
+        const T* Xs = tiles + buf * L::TILE;
+        const T* Ys = Xs + 64 * XS;
+        const T* Zs = Ys + 64 * XS;
         if (have_next) load_block(REVERSE ? t - 1 : t + 1);
 
-        // ---- 1. S^T tiles for tokens i in [16w, 16w+16) ----------------------
-        {
-            f32x4 sacc[4];
+        // =================== phase 1 =========================================
+        if (!state_role) {
+            // S^T tiles of this wave -> masked, decayed P[i][j]
+            f32x4 sacc[3];
 #pragma unroll
-            for (int jt = 0; jt < 4; ++jt) sacc[jt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            for (int sl = 0; sl < 3; ++sl) sacc[sl] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            const T* xa = Xs + (16 * itA + r) * XS + 8 * g;
+            const T* y0 = Ys + (16 * jt0 + r) * XS + 8 * g;
+            if (itB >= 0) {
+                const T* xb = Xs + (16 * itB + r) * XS + 8 * g;
+                const T* y1 = Ys + (16 * jt1 + r) * XS + 8 * g;
+                const T* y2 = Ys + (16 * jt2 + r) * XS + 8 * g;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const V8 bx = *reinterpret_cast<const V8*>(Xs + (16 * w + r) * XS + 32 * ks + 8 * g);
-#pragma unroll
-                for (int jt = 0; jt < 4; ++jt) {
-                    if (jt >= jlo && jt <= jhi) {
-                        const V8 ay = *reinterpret_cast<const V8*>(Ys + (16 * jt + r) * XS + 32 * ks + 8 * g);
-                        sacc[jt] = M::mma(ay, bx, sacc[jt]);
-                    }
+                for (int ks = 0; ks < KS; ++ks) {
+                    const V8 bxa = *reinterpret_cast<const V8*>(xa + 32 * ks);
+                    const V8 bxb = *reinterpret_cast<const V8*>(xb + 32 * ks);
+                    sacc[0] = M::mma(*reinterpret_cast<const V8*>(y0 + 32 * ks), bxa, sacc[0]);
+                    sacc[1] = M::mma(*reinterpret_cast<const V8*>(y1 + 32 * ks), bxb, sacc[1]);
+                    sacc[2] = M::mma(*reinterpret_cast<const V8*>(y2 + 32 * ks), bxb, sacc[2]);
                 }
-            }
+            } else {
 #pragma unroll
-            for (int jt = 0; jt < 4; ++jt) {
-                if (jt >= jlo && jt <= jhi) {
-                    V4 p;
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[jt][v] * dfac[jt][v]);
-                    *reinterpret_cast<V4*>(Ps + (16 * w + r) * ZS + 16 * jt + 4 * g) = p;
-                }
+                for (int ks = 0; ks < KS; ++ks)
+                    sacc[0] = M::mma(*reinterpret_cast<const V8*>(y0 + 32 * ks),
+                                     *reinterpret_cast<const V8*>(xa + 32 * ks), sacc[0]);
             }
-        }
-        __syncthreads();
-
-        if (wave_active) {
-            // z^T fragments: rows (tokens) 32ks + 8g + u, column 16w + r
-            V8 zf[2];
+            {
+                V4 p;
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                const T* pz = Zs + (32 * ks + 8 * g + (r >> 2)) * ZS + 16 * w + 4 * (r & 3);
-                zf[ks] = cat<V8, V4>(lds_tr4<V4>(pz), lds_tr4<V4>(pz + 4 * ZS));
+                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[0][v] * dfac[0][v]);
+                *reinterpret_cast<V4*>(Ps + (16 * itA + r) * ZS + 16 * jt0 + 4 * g) = p;
             }
-            // ---- 2a. inter-block term: out^T = state^T x^T -------------------
+            if (itB >= 0) {
+                V4 p;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[1][v] * dfac[1][v]);
+                *reinterpret_cast<V4*>(Ps + (16 * itB + r) * ZS + 16 * jt1 + 4 * g) = p;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[2][v] * dfac[2][v]);
+                *reinterpret_cast<V4*>(Ps + (16 * itB + r) * ZS + 16 * jt2 + 4 * g) = p;
+            }
+        } else if (cols_active) {
+            // inter-block term: out^T[c][i] = Lout[i] * sum_k state[k][c] x[i][k]
             V8 sb[KS];
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
@@ -242,77 +289,108 @@ __global__ __launch_bounds__(256, 1) void la_sweep_kernel(SweepArgs a) {
             }
             f32x4 oacc[4];
 #pragma unroll
-            for (int i4 = 0; i4 < 4; ++i4) {
-                oacc[i4] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            for (int i4 = 0; i4 < 4; ++i4) oacc[i4] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
+            for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) {
                     const T* px = Xs + (16 * i4 + r) * XS + 32 * ks + 4 * g;
                     const V8 bx = cat<V8, V4>(*reinterpret_cast<const V4*>(px), *reinterpret_cast<const V4*>(px + 16));
                     oacc[i4] = M::mma(sb[ks], bx, oacc[i4]);
                 }
+            }
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
                 if (DECAY) {
 #pragma unroll
                     for (int v = 0; v < 4; ++v) oacc[i4][v] *= ofac[i4];
                 }
-            }
-            // ---- 2b. intra-block term: out^T += z^T P^T ----------------------
-#pragma unroll
-            for (int i4 = 0; i4 < 4; ++i4) {
-#pragma unroll
-                for (int ks = 0; ks < 2; ++ks) {
-                    const bool need = REVERSE ? (ks >= i4 / 2) : (ks <= i4 / 2);
-                    if (need) {
-                        const V8 bp = *reinterpret_cast<const V8*>(Ps + (16 * i4 + r) * ZS + 32 * ks + 8 * g);
-                        oacc[i4] = M::mma(zf[ks], bp, oacc[i4]);
-                    }
-                }
-            }
-            // ---- store out[token][16w + 4g .. +3] ----------------------------
-            const int col = col0 + 16 * w + 4 * g;
-#pragma unroll
-            for (int i4 = 0; i4 < 4; ++i4) {
-                const int64_t tok = t * 64 + 16 * i4 + r;
-                if (tok < n && col < dv) {
-                    V4 o;
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) o[v] = (T)oacc[i4][v];
-                    *reinterpret_cast<V4*>(og + tok * dv + col) = o;
-                }
-            }
-            // ---- 3. state = lam^64 state + y^T (z * Lupd) ---------------------
-            if (have_next) {
-                if (DECAY) {
-#pragma unroll
-                    for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) zf[ks][u] = (T)((float)zf[ks][u] * zfac[ks][u]);
-#pragma unroll
-                    for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-                        for (int v = 0; v < 4; ++v) st[kt][v] *= lamB;
-                }
-#pragma unroll
-                for (int kt = 0; kt < KT; ++kt) {
-#pragma unroll
-                    for (int ks = 0; ks < 2; ++ks) {
-                        const T* py = Ys + (32 * ks + 8 * g + (r >> 2)) * XS + 16 * kt + 4 * (r & 3);
-                        const V8 ay = cat<V8, V4>(lds_tr4<V4>(py), lds_tr4<V4>(py + 4 * XS));
-                        st[kt] = M::mma(ay, zf[ks], st[kt]);
-                    }
-                }
+                Ob[(w * 4 + i4) * 64 + lane] = oacc[i4];
             }
         }
         __syncthreads();
-        if (have_next) {
-            stage_block();
+
+        // =================== phase 2 =========================================
+        if (!state_role) {
+            if (cols_active) {
+                // out^T = inter + z^T P^T, then store out[token][16w + 4g .. +3]
+                V8 zf[2];
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) {
+                    const T* pz = Zs + (32 * ks + 8 * g + (r >> 2)) * ZS + 16 * w + 4 * (r & 3);
+                    zf[ks] = cat<V8, V4>(lds_tr4<V4>(pz), lds_tr4<V4>(pz + 4 * ZS));
+                }
+                f32x4 oacc[4];
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) oacc[i4] = Ob[(w * 4 + i4) * 64 + lane];
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) {
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks) {
+                        const bool need = REVERSE ? (ks >= i4 / 2) : (ks <= i4 / 2);
+                        if (need) {
+                            const V8 bp = *reinterpret_cast<const V8*>(Ps + (16 * i4 + r) * ZS + 32 * ks + 8 * g);
+                            oacc[i4] = M::mma(zf[ks], bp, oacc[i4]);
+                        }
+                    }
+                }
+                const int col = col0 + 16 * w + 4 * g;
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) {
+                    const int64_t tok = t * 64 + 16 * i4 + r;
+                    if (tok < n && col < dv) {
+                        V4 o;
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) o[v] = (T)oacc[i4][v];
+                        *reinterpret_cast<V4*>(og + tok * dv + col) = o;
+                    }
+                }
+            }
+        } else if (cols_active && have_next) {
+            // state = lam^64 state + y^T (z * Lupd)
+            V8 zf[2];
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                const T* pz = Zs + (32 * ks + 8 * g + (r >> 2)) * ZS + 16 * w + 4 * (r & 3);
+                zf[ks] = cat<V8, V4>(lds_tr4<V4>(pz), lds_tr4<V4>(pz + 4 * ZS));
+            }
+            if (DECAY) {
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) zf[ks][u] = (T)((float)zf[ks][u] * zfac[ks][u]);
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) st[kt][v] *= lamB;
+            }
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) {
+                    const T* py = Ys + (32 * ks + 8 * g + (r >> 2)) * XS + 16 * kt + 4 * (r & 3);
+                    const V8 ay = cat<V8, V4>(lds_tr4<V4>(py), lds_tr4<V4>(py + 4 * XS));
+                    st[kt] = M::mma(ay, zf[ks], st[kt]);
+                }
+            }
+        }
+        if (NBUF == 2) {
+            if (have_next) stage_block((int)((it + 1) & 1));
             __syncthreads();
+        } else {
+            __syncthreads();
+            if (have_next) {
+                stage_block(0);
+                __syncthreads();
+            }
         }
     }
 }
 
 template <typename T, int DKP, bool REVERSE, bool DECAY>
 static int launch_one(const SweepArgs& a, hipStream_t st) {
-    constexpr size_t lds = (size_t)(2 * 64 * (DKP + 8) + 2 * 64 * 72) * sizeof(T);
+    constexpr size_t lds = SweepLds<DKP>::bytes(sizeof(T));
+    static_assert(lds <= 160 * 1024, "LDS budget");
     auto kern = la_sweep_kernel<T, DKP, REVERSE, DECAY>;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -321,7 +399,7 @@ static int launch_one(const SweepArgs& a, hipStream_t st) {
     }
     const int units8 = (a.bh + 7) / 8 * 8;
     const unsigned grid = (unsigned)(units8 * a.nslice);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, a);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, st, a);
     return (int)hipGetLastError();
 }
 
@@ -329,7 +407,6 @@ template <typename T, bool REVERSE>
 static int launch_dir(const SweepArgs& a, hipStream_t st) {
     const bool decay = a.s != nullptr;
 #define LA_GO(DKP) (decay ? launch_one<T, DKP, REVERSE, true>(a, st) : launch_one<T, DKP, REVERSE, false>(a, st))
-    if (a.dk <= 32) return LA_GO(32);
     if (a.dk <= 64) return LA_GO(64);
     if (a.dk <= 128) return LA_GO(128);
     if (a.dk <= 192) return LA_GO(192);
