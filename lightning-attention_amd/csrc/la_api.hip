@@ -1,10 +1,14 @@
 // extern "C" entry points of the attention path (see include/lightning_attn_hip.h).
+#include <stdlib.h>
+
 #include "la_common.h"
 #include "lightning_attn_hip.h"
 
 namespace la {
 int sweep(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h, int64_t n,
           int64_t dk, int64_t dv, int dtype, bool reverse, hipStream_t st);
+int sweep32(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h, int64_t n,
+            int64_t dk, int64_t dv, int dtype, bool reverse, hipStream_t st);
 int sweep_f32(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
               int64_t n, int64_t dk, int64_t dv, bool reverse, hipStream_t st);
 
@@ -12,6 +16,10 @@ int sweep_f32(const void* x, const void* y, const void* z, void* out, const floa
 static int run(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
                int64_t n, int64_t dk, int64_t dv, int dtype, bool reverse, hipStream_t st) {
     if (dtype == LA_FP32) return sweep_f32(x, y, z, out, s, bh, h, n, dk, dv, reverse, st);
+    // contraction dims up to 128 run the 32x32x16 kernel (two state waves + three score
+    // waves); wider ones the 16x16x32 kernel.  LA_SWEEP_WIDE=1 forces the latter (testing).
+    static const bool force_wide = [] { const char* e = getenv("LA_SWEEP_WIDE"); return e && e[0] == '1'; }();
+    if (dk <= 128 && !force_wide) return sweep32(x, y, z, out, s, bh, h, n, dk, dv, dtype, reverse, st);
     return sweep(x, y, z, out, s, bh, h, n, dk, dv, dtype, reverse, st);
 }
 
@@ -19,7 +27,9 @@ static inline bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) 
 
 static int check_dims(int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype) {
     if (b < 0 || h <= 0 || n < 0 || d <= 0 || e <= 0) return LA_E_SHAPE;
-    if (b * h > 0x7fffffffLL / 64 || n > (1LL << 40)) return LA_E_SHAPE;
+    if (b * h > 0x7fffffffLL / 64) return LA_E_SHAPE;
+    // the kernels address one (batch, head) slice with 32-bit byte offsets below 2 GiB
+    if (n * (d > e ? d : e) * 4 >= (1LL << 31)) return LA_E_SHAPE;
     if (!la_supported(d, e, dtype)) return LA_E_UNSUPPORTED;
     return LA_OK;
 }

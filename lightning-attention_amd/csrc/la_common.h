@@ -13,7 +13,25 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
 
+typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
+typedef __attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned u32x2;
+
 constexpr int kWave = 64;
+
+// Raw buffer access with hardware bounds checking: a load whose byte offset lies at
+// or beyond `bytes` returns zeros and such a store is dropped, so ragged tails need
+// no branches.  kOob is an offset that is out of range for every buffer used here
+// (all are smaller than 2 GiB).
+constexpr unsigned kOob = 0x80000000u;
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ u32x4 buf_load16(__amdgpu_buffer_rsrc_t r, unsigned off) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+}
+__device__ __forceinline__ void buf_store8(__amdgpu_buffer_rsrc_t r, unsigned off, u32x2 v) {
+    __builtin_amdgcn_raw_buffer_store_b64(v, r, off, 0, 0);
+}
 
 template <typename T>
 struct ElemTraits;
