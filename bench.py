@@ -102,7 +102,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--no-sweep", action="store_true", help="skip the n sweep and SRMSNorm timings")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the fwd/bwd split and the n sweep")
+    ap.add_argument("--no-srms", action="store_true", help="skip the SRMSNorm timings")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU part (every (batch, head) sequence is "
@@ -204,11 +205,12 @@ def main():
         del o
         sweep = {}
         for n in (512, 1024, 2048, 4096, 8192, 16384, 32768):
-            del q, k, v, do
+            q = k = v = do = None
             q, k, v, do = inputs(n)
             sweep[str(n)] = round(event_ms(step, 10 if n >= 16384 else 20), 4)
         out["n_sweep_fwd_bwd_ms"] = sweep
-        del q, k, v, do
+    del q, k, v, do
+    if not args.no_srms:
         # SRMSNorm, config 5: [32768, 4096] bf16, 1 % outliers x50
         rows, cols = 32768, 4096
         x = torch.randn(rows, cols, device=dev)

@@ -1,14 +1,10 @@
 // extern "C" entry points of the attention path (see include/lightning_attn_hip.h).
-#include <stdlib.h>
-
 #include "la_common.h"
 #include "lightning_attn_hip.h"
 
 namespace la {
 int sweep(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h, int64_t n,
           int64_t dk, int64_t dv, int dtype, bool reverse, hipStream_t st);
-int sweep32(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h, int64_t n,
-            int64_t dk, int64_t dv, int dtype, bool reverse, hipStream_t st);
 int sweep_f32(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
               int64_t n, int64_t dk, int64_t dv, bool reverse, hipStream_t st);
 
@@ -16,10 +12,6 @@ int sweep_f32(const void* x, const void* y, const void* z, void* out, const floa
 static int run(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
                int64_t n, int64_t dk, int64_t dv, int dtype, bool reverse, hipStream_t st) {
     if (dtype == LA_FP32) return sweep_f32(x, y, z, out, s, bh, h, n, dk, dv, reverse, st);
-    // contraction dims up to 128 run the 32x32x16 kernel (two state waves + three score
-    // waves); wider ones the 16x16x32 kernel.  LA_SWEEP_WIDE=1 forces the latter (testing).
-    static const bool force_wide = [] { const char* e = getenv("LA_SWEEP_WIDE"); return e && e[0] == '1'; }();
-    if (dk <= 128 && !force_wide) return sweep32(x, y, z, out, s, bh, h, n, dk, dv, dtype, reverse, st);
     return sweep(x, y, z, out, s, bh, h, n, dk, dv, dtype, reverse, st);
 }
 

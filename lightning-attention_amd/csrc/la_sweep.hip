@@ -129,10 +129,11 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
     const int lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int64_t n = a.n;
     const int dk = a.dk, dv = a.dv;
-    const T* xg = static_cast<const T*>(a.x) + (int64_t)unit * n * dk;
-    const T* yg = static_cast<const T*>(a.y) + (int64_t)unit * n * dk;
-    const T* zg = static_cast<const T*>(a.z) + (int64_t)unit * n * dv;
-    T* og = static_cast<T*>(a.out) + (int64_t)unit * n * dv;
+    // one bounds-checked buffer per (batch, head) slice: rows >= n read as zero / are not written
+    const __amdgpu_buffer_rsrc_t xb = make_rsrc(static_cast<const T*>(a.x) + (int64_t)unit * n * dk, (unsigned)(n * dk * sizeof(T)));
+    const __amdgpu_buffer_rsrc_t yb = make_rsrc(static_cast<const T*>(a.y) + (int64_t)unit * n * dk, (unsigned)(n * dk * sizeof(T)));
+    const __amdgpu_buffer_rsrc_t zb = make_rsrc(static_cast<const T*>(a.z) + (int64_t)unit * n * dv, (unsigned)(n * dv * sizeof(T)));
+    const __amdgpu_buffer_rsrc_t ob = make_rsrc(static_cast<T*>(a.out) + (int64_t)unit * n * dv, (unsigned)(n * dv * sizeof(T)));
     const int col0 = slice * 64;
     const bool cols_active = (col0 + 16 * w) < dv;
 
@@ -185,22 +186,23 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
     for (int kt = 0; kt < KT; ++kt) st[kt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
     const int64_t nblk = (n + 63) / 64;
-    uint4 xr[XC], yr[XC], zr;
+    u32x4 xr[XC], yr[XC], zr;
 
     auto load_block = [&](int64_t t) {
-        const int64_t tok0 = t * 64;
+        const unsigned tok0 = (unsigned)(t * 64);
 #pragma unroll
         for (int u = 0; u < XC; ++u) {
             const int c = tid + 512 * u;
             const int row = c / (DKP / 8), col = (c % (DKP / 8)) * 8;
-            const bool ok = (tok0 + row < n) && (col < dk);
-            xr[u] = ok ? *reinterpret_cast<const uint4*>(xg + (tok0 + row) * dk + col) : make_uint4(0, 0, 0, 0);
-            yr[u] = ok ? *reinterpret_cast<const uint4*>(yg + (tok0 + row) * dk + col) : make_uint4(0, 0, 0, 0);
+            // columns dk..DKP-1 are zero padding
+            const unsigned off = col < dk ? ((tok0 + row) * (unsigned)dk + col) * (unsigned)sizeof(T) : kOob;
+            xr[u] = buf_load16(xb, off);
+            yr[u] = buf_load16(yb, off);
         }
         {
             const int row = tid / 8, col = (tid % 8) * 8;
-            const bool ok = (tok0 + row < n) && (col0 + col < dv);
-            zr = ok ? *reinterpret_cast<const uint4*>(zg + (tok0 + row) * dv + col0 + col) : make_uint4(0, 0, 0, 0);
+            const unsigned off = (col0 + col < dv) ? ((tok0 + row) * (unsigned)dv + col0 + col) * (unsigned)sizeof(T) : kOob;
+            zr = buf_load16(zb, off);
         }
     };
     auto stage_block = [&](int buf) {
@@ -211,12 +213,12 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
         for (int u = 0; u < XC; ++u) {
             const int c = tid + 512 * u;
             const int row = c / (DKP / 8), col = (c % (DKP / 8)) * 8;
-            *reinterpret_cast<uint4*>(Xd + row * XS + col) = xr[u];
-            *reinterpret_cast<uint4*>(Yd + row * XS + col) = yr[u];
+            *reinterpret_cast<u32x4*>(Xd + row * XS + col) = xr[u];
+            *reinterpret_cast<u32x4*>(Yd + row * XS + col) = yr[u];
         }
         {
             const int row = tid / 8, col = (tid % 8) * 8;
-            *reinterpret_cast<uint4*>(Zd + row * ZS + col) = zr;
+            *reinterpret_cast<u32x4*>(Zd + row * ZS + col) = zr;
         }
     };
 
@@ -337,13 +339,12 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
                 const int col = col0 + 16 * w + 4 * g;
 #pragma unroll
                 for (int i4 = 0; i4 < 4; ++i4) {
-                    const int64_t tok = t * 64 + 16 * i4 + r;
-                    if (tok < n && col < dv) {
-                        V4 o;
+                    const unsigned tok = (unsigned)(t * 64) + 16 * i4 + r;
+                    V4 o;
 #pragma unroll
-                        for (int v = 0; v < 4; ++v) o[v] = (T)oacc[i4][v];
-                        *reinterpret_cast<V4*>(og + tok * dv + col) = o;
-                    }
+                    for (int v = 0; v < 4; ++v) o[v] = (T)oacc[i4][v];
+                    const unsigned off = col < dv ? (tok * (unsigned)dv + col) * (unsigned)sizeof(T) : kOob;
+                    buf_store8(ob, off, __builtin_bit_cast(u32x2, o));
                 }
             }
         } else if (cols_active && have_next) {
