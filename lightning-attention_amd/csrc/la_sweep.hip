@@ -93,8 +93,14 @@ __device__ __constant__ const TileDeal kDeal[4] = {
 
 template <int DKP>
 struct SweepLds {
-    static constexpr int XS = DKP + 8;  // row stride (elements) of the x / y tiles
-    static constexpr int ZS = 64 + 8;   // row stride of the z slice and the P tile
+#ifndef LA_XPAD
+#define LA_XPAD 8
+#endif
+#ifndef LA_ZPAD
+#define LA_ZPAD 8
+#endif
+    static constexpr int XS = DKP + LA_XPAD;  // row stride (elements) of the x / y tiles
+    static constexpr int ZS = 64 + LA_ZPAD;   // row stride of the z slice and the P tile
     static constexpr int NBUF = DKP <= 192 ? 2 : 1;
     static constexpr int TILE = 2 * 64 * XS + 64 * ZS;  // elements of one x+y+z buffer
     static constexpr size_t bytes(size_t elt) { return (size_t)(NBUF * TILE + 64 * ZS) * elt + 4 * 4 * 64 * 16; }
