@@ -23,6 +23,8 @@
 // contraction index on the B side.  Transposed operands (y^T, z^T) come from the
 // LDS transpose read ds_read_b64_tr_b16.  x/y/z tiles are double-buffered in LDS
 // (global -> registers one block ahead -> LDS), two barriers per block.
+#include <stdlib.h>
+
 #include "la_common.h"
 #include "lightning_attn_hip.h"
 
@@ -36,6 +38,8 @@ struct SweepArgs {
     const float* s; // h decay rates or nullptr
     int64_t n;
     int dk, dv, h, bh, nslice;
+    int nchunk;          // sequence chunks per (batch, head, slice); 1 = one workgroup walks the whole sequence
+    int chunk_start[9];  // first 64-token block (in walk order) of each chunk; chunk_start[nchunk] = number of blocks
 };
 
 template <typename T>
@@ -124,8 +128,10 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
     // Workgroups are dealt round-robin to the 8 XCDs by linear id; keep the
     // column slices of one head on one XCD so their x / y re-reads share an L2.
     const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-    const int unit = xcd + 8 * (local / a.nslice);
-    const int slice = local % a.nslice;
+    const int per_unit = a.nslice * a.nchunk;
+    const int unit = xcd + 8 * (local / per_unit);
+    const int slice = (local % per_unit) % a.nslice;
+    const int chunk = (local % per_unit) / a.nslice;
     if (unit >= a.bh) return;
 
     const int tid = threadIdx.x;
@@ -192,9 +198,15 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
     for (int kt = 0; kt < KT; ++kt) st[kt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
     const int64_t nblk = (n + 63) / 64;
+    // Sequence chunking (chunk-parallel variant): this workgroup produces the blocks
+    // [it_first, it_end) of the walk.  It first runs over the blocks before it_first with the
+    // state update only ("warm-up": y and z are read, nothing is written) to rebuild the state
+    // its chunk starts from; there is no hand-off between workgroups and no workspace.
+    const int64_t it_first = a.chunk_start[chunk];
+    const int64_t it_end = a.chunk_start[chunk + 1];
     u32x4 xr[XC], yr[XC], zr;
 
-    auto load_block = [&](int64_t t) {
+    auto load_block = [&](int64_t t, bool need_x) {
         const unsigned tok0 = (unsigned)(t * 64);
 #pragma unroll
         for (int u = 0; u < XC; ++u) {
@@ -202,7 +214,7 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
             const int row = c / (DKP / 8), col = (c % (DKP / 8)) * 8;
             // columns dk..DKP-1 are zero padding
             const unsigned off = col < dk ? ((tok0 + row) * (unsigned)dk + col) * (unsigned)sizeof(T) : kOob;
-            xr[u] = buf_load16(xb, off);
+            xr[u] = buf_load16(xb, need_x ? off : kOob);
             yr[u] = buf_load16(yb, off);
         }
         {
@@ -230,21 +242,24 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
 
     // zero P once: tiles on the masked side of the diagonal are never written
     for (int c = tid; c < 64 * ZS / 8; c += 512) reinterpret_cast<uint4*>(Ps)[c] = make_uint4(0, 0, 0, 0);
-    load_block(REVERSE ? nblk - 1 : 0);
+    load_block(REVERSE ? nblk - 1 : 0, it_first == 0);
     stage_block(0);
     __syncthreads();
 
-    for (int64_t it = 0; it < nblk; ++it) {
+    for (int64_t it = 0; it < it_end; ++it) {
         const int64_t t = REVERSE ? nblk - 1 - it : it;
-        const bool have_next = it + 1 < nblk;
+        const bool have_next = it + 1 < it_end;
+        const bool warm = it < it_first;  // warm-up block: state update only
         const int buf = NBUF == 2 ? (int)(it & 1) : 0;
         const T* Xs = tiles + buf * L::TILE;
         const T* Ys = Xs + 64 * XS;
         const T* Zs = Ys + 64 * XS;
-        if (have_next) load_block(REVERSE ? t - 1 : t + 1);
+        if (have_next) load_block(REVERSE ? t - 1 : t + 1, it + 1 >= it_first);
 
         // =================== phase 1 =========================================
-        if (!state_role) {
+        if (warm) {
+            // nothing: x is not needed and no output is produced
+        } else if (!state_role) {
             // S^T tiles of this wave -> masked, decayed P[i][j]
             f32x4 sacc[3];
 #pragma unroll
@@ -316,11 +331,11 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
                 Ob[(w * 4 + i4) * 64 + lane] = oacc[i4];
             }
         }
-        __syncthreads();
+        if (!warm) __syncthreads();  // warm-up blocks share nothing between the two phases
 
         // =================== phase 2 =========================================
         if (!state_role) {
-            if (cols_active) {
+            if (cols_active && !warm) {
                 // out^T = inter + z^T P^T, then store out[token][16w + 4g .. +3]
                 V8 zf[2];
 #pragma unroll
@@ -405,7 +420,7 @@ static int launch_one(const SweepArgs& a, hipStream_t st) {
         if (e != hipSuccess) return (int)e;
     }
     const int units8 = (a.bh + 7) / 8 * 8;
-    const unsigned grid = (unsigned)(units8 * a.nslice);
+    const unsigned grid = (unsigned)(units8 * a.nslice * a.nchunk);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, st, a);
     return (int)hipGetLastError();
 }
@@ -421,6 +436,50 @@ static int launch_dir(const SweepArgs& a, hipStream_t st) {
 #undef LA_GO
 }
 
+// Sequence chunks per (batch, head, slice).  With few sequences a single sweep per sequence
+// leaves most of the 256 CUs idle; the walk is then cut into up to 8 chunks whose workgroups
+// rebuild their incoming state themselves.  A warm-up block costs about half a full block, so
+// chunk lengths shrink geometrically (len_c ~ (1 - rho)^c, rho = 0.5) to make all workgroups
+// finish together.  LA_SWEEP_CHUNKS=<C> overrides the count.
+static void choose_chunks(SweepArgs& a) {
+    const char* env = getenv("LA_SWEEP_CHUNKS");  // read per call so that tests can vary it
+    const int forced = env ? atoi(env) : 0;
+    static const int cus = [] {
+        int dev = 0, n = 256;
+        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+        return n > 0 ? n : 256;
+    }();
+    const int64_t nblk = (a.n + 63) / 64;
+    const int64_t wgs = (int64_t)((a.bh + 7) / 8 * 8) * a.nslice;
+    int64_t c = 1;
+    if (forced > 0) c = forced;
+    else if (wgs * 2 <= cus && nblk >= 8) {
+        c = cus / wgs;
+        if (c > nblk / 4) c = nblk / 4;
+    }
+    if (c > 8) c = 8;
+    if (c > nblk) c = nblk;
+    if (c < 1) c = 1;
+    // geometric lengths, at least one block each, summing to nblk
+    const double rho = 0.5;
+    double wsum = 0.0, wgt = 1.0;
+    for (int i = 0; i < c; ++i) { wsum += wgt; wgt *= 1.0 - rho; }
+    int64_t start = 0;
+    wgt = 1.0;
+    for (int i = 0; i < c; ++i) {
+        a.chunk_start[i] = (int)start;
+        int64_t len = (int64_t)((double)nblk * wgt / wsum + 0.5);
+        const int64_t left_after = c - 1 - i;
+        if (len < 1) len = 1;
+        if (start + len > nblk - left_after) len = nblk - left_after - start;
+        start += len;
+        wgt *= 1.0 - rho;
+    }
+    a.nchunk = (int)c;
+    a.chunk_start[c] = (int)nblk;
+    for (int i = (int)c + 1; i < 9; ++i) a.chunk_start[i] = (int)nblk;
+}
+
 // x,y: (bh,n,dk)  z,out: (bh,n,dv)
 int sweep(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h, int64_t n,
           int64_t dk, int64_t dv, int dtype, bool reverse, hipStream_t st) {
@@ -428,6 +487,7 @@ int sweep(const void* x, const void* y, const void* z, void* out, const float* s
     a.x = x; a.y = y; a.z = z; a.out = out; a.s = s;
     a.n = n; a.dk = (int)dk; a.dv = (int)dv; a.h = (int)h; a.bh = (int)bh;
     a.nslice = (int)((dv + 63) / 64);
+    choose_chunks(a);
     if (dtype == LA_BF16) return reverse ? launch_dir<__bf16, true>(a, st) : launch_dir<__bf16, false>(a, st);
     if (dtype == LA_FP16) return reverse ? launch_dir<_Float16, true>(a, st) : launch_dir<_Float16, false>(a, st);
     return LA_E_UNSUPPORTED;

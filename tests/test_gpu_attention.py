@@ -171,6 +171,28 @@ def test_wide_features_are_split_by_the_interface():
     check(run_hip(qf, kf, vf, s, dof), want, torch.float32, "wide fp32")
 
 
+@pytest.mark.parametrize("b, h, n, d, e", [(1, 2, 4096, 128, 64), (2, 3, 1000, 64, 128), (1, 1, 1500, 192, 72)])
+def test_sequence_chunking_is_exact(b, h, n, d, e, monkeypatch):
+    """Few sequences: the walk is cut into chunks whose workgroups rebuild their incoming state
+    (the chunk-parallel path).  Every chunk count must give bit-identical results, and they must
+    match the oracle."""
+    q, k, v, do = make_inputs(b, h, n, d, e, torch.bfloat16, 1.0, seed=n)
+    s = _build_slope_tensor(h)
+    outs = {}
+    for chunks in ("1", "2", "3", "8", None):  # None = the library's own choice
+        if chunks is None:
+            monkeypatch.delenv("LA_SWEEP_CHUNKS", raising=False)
+        else:
+            monkeypatch.setenv("LA_SWEEP_CHUNKS", chunks)
+        outs[chunks] = run_hip(q, k, v, s, do)
+    monkeypatch.delenv("LA_SWEEP_CHUNKS", raising=False)
+    for chunks in ("2", "3", "8", None):
+        for a, c in zip(outs["1"], outs[chunks]):
+            assert torch.equal(a, c), chunks
+    want = oracle.linear_attn_fwd_bwd(q, k, v, s, do, torch.float32)
+    check(outs[None], want, torch.bfloat16, "chunked %s" % ((b, h, n, d, e),))
+
+
 def test_deterministic():
     q, k, v, do = make_inputs(2, 8, 1000, 128, 128, torch.bfloat16, 1.0)
     s = _build_slope_tensor(8)
