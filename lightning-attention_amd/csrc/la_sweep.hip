@@ -204,9 +204,19 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
     // its chunk starts from; there is no hand-off between workgroups and no workspace.
     const int64_t it_first = a.chunk_start[chunk];
     const int64_t it_end = a.chunk_start[chunk + 1];
-    u32x4 xr[XC], yr[XC], zr;
+    // Two register sets of prefetched tiles (feature dims up to 128; wider ones have no registers
+    // to spare and keep one): while block `it` is worked on, block it+1 sits in LDS and blocks
+    // it+2, it+3 are in flight from memory (one block of prefetch does not cover the memory
+    // latency under load).
+    constexpr int NSET = DKP <= 128 ? 2 : 1;
+    u32x4 xrA[XC], yrA[XC], zrA, xrB[XC], yrB[XC], zrB;
 
-    auto load_block = [&](int64_t t, bool need_x) {
+    // Fetches block number b of the walk.  Blocks at or beyond it_end, and the x tile of warm-up
+    // blocks, are fetched at the out-of-range offset: zeros, no memory traffic, and the sequence of
+    // loads is the same on every path.
+    auto load_block = [&](int64_t b, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4& zr) {
+        const int64_t t = REVERSE ? nblk - 1 - b : b;
+        const bool valid = b < it_end, need_x = valid && b >= it_first;
         const unsigned tok0 = (unsigned)(t * 64);
 #pragma unroll
         for (int u = 0; u < XC; ++u) {
@@ -215,15 +225,15 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
             // columns dk..DKP-1 are zero padding
             const unsigned off = col < dk ? ((tok0 + row) * (unsigned)dk + col) * (unsigned)sizeof(T) : kOob;
             xr[u] = buf_load16(xb, need_x ? off : kOob);
-            yr[u] = buf_load16(yb, off);
+            yr[u] = buf_load16(yb, valid ? off : kOob);
         }
         {
             const int row = tid / 8, col = (tid % 8) * 8;
             const unsigned off = (col0 + col < dv) ? ((tok0 + row) * (unsigned)dv + col0 + col) * (unsigned)sizeof(T) : kOob;
-            zr = buf_load16(zb, off);
+            zr = buf_load16(zb, valid ? off : kOob);
         }
     };
-    auto stage_block = [&](int buf) {
+    auto stage_block = [&](int buf, const u32x4 (&xr)[XC], const u32x4 (&yr)[XC], const u32x4& zr) {
         T* Xd = tiles + buf * L::TILE;
         T* Yd = Xd + 64 * XS;
         T* Zd = Yd + 64 * XS;
@@ -242,11 +252,14 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
 
     // zero P once: tiles on the masked side of the diagonal are never written
     for (int c = tid; c < 64 * ZS / 8; c += 512) reinterpret_cast<uint4*>(Ps)[c] = make_uint4(0, 0, 0, 0);
-    load_block(REVERSE ? nblk - 1 : 0, it_first == 0);
-    stage_block(0);
+    load_block(0, xrA, yrA, zrA);
+    if (NSET == 2) load_block(1, xrB, yrB, zrB);
+    stage_block(0, xrA, yrA, zrA);
+    load_block(NSET == 2 ? 2 : 1, xrA, yrA, zrA);
     __syncthreads();
 
-    for (int64_t it = 0; it < it_end; ++it) {
+    // One block of the walk.  `xr, yr, zr` hold block it+1 on entry and block it+3 on exit.
+    auto block_body = [&](const int64_t it, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4& zr) {
         const int64_t t = REVERSE ? nblk - 1 - it : it;
         const bool have_next = it + 1 < it_end;
         const bool warm = it < it_first;  // warm-up block: state update only
@@ -254,7 +267,12 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
         const T* Xs = tiles + buf * L::TILE;
         const T* Ys = Xs + 64 * XS;
         const T* Zs = Ys + 64 * XS;
-        if (have_next) load_block(REVERSE ? t - 1 : t + 1, it + 1 >= it_first);
+        if (NSET == 2) {
+            // publish block it+1 (its LDS buffer was last read in block it-1) and refill the
+            // registers with block it+3: both overlap the matrix work below
+            stage_block((int)((it + 1) & 1), xr, yr, zr);
+            load_block(it + 3, xr, yr, zr);
+        }
 
         // =================== phase 1 =========================================
         if (warm) {
@@ -266,23 +284,47 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
             for (int sl = 0; sl < 3; ++sl) sacc[sl] = (f32x4){0.f, 0.f, 0.f, 0.f};
             const T* xa = Xs + (16 * itA + r) * XS + 8 * g;
             const T* y0 = Ys + (16 * jt0 + r) * XS + 8 * g;
+            // all fragment reads of a batch are issued before its MFMAs (the scheduler otherwise
+            // sinks each read next to its use and the wave pays one LDS round trip per MFMA)
+            constexpr int SB = KS <= 4 ? KS : 2;  // contraction steps per batch
             if (itB >= 0) {
                 const T* xb = Xs + (16 * itB + r) * XS + 8 * g;
                 const T* y1 = Ys + (16 * jt1 + r) * XS + 8 * g;
                 const T* y2 = Ys + (16 * jt2 + r) * XS + 8 * g;
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    const V8 bxa = *reinterpret_cast<const V8*>(xa + 32 * ks);
-                    const V8 bxb = *reinterpret_cast<const V8*>(xb + 32 * ks);
-                    sacc[0] = M::mma(*reinterpret_cast<const V8*>(y0 + 32 * ks), bxa, sacc[0]);
-                    sacc[1] = M::mma(*reinterpret_cast<const V8*>(y1 + 32 * ks), bxb, sacc[1]);
-                    sacc[2] = M::mma(*reinterpret_cast<const V8*>(y2 + 32 * ks), bxb, sacc[2]);
+                for (int k0 = 0; k0 < KS; k0 += SB) {
+                    V8 fxa[SB], fxb[SB], fy0[SB], fy1[SB], fy2[SB];
+#pragma unroll
+                    for (int ks = 0; ks < SB; ++ks) {
+                        fxa[ks] = *reinterpret_cast<const V8*>(xa + 32 * (k0 + ks));
+                        fy0[ks] = *reinterpret_cast<const V8*>(y0 + 32 * (k0 + ks));
+                        fxb[ks] = *reinterpret_cast<const V8*>(xb + 32 * (k0 + ks));
+                        fy1[ks] = *reinterpret_cast<const V8*>(y1 + 32 * (k0 + ks));
+                        fy2[ks] = *reinterpret_cast<const V8*>(y2 + 32 * (k0 + ks));
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int ks = 0; ks < SB; ++ks) {
+                        sacc[0] = M::mma(fy0[ks], fxa[ks], sacc[0]);
+                        sacc[1] = M::mma(fy1[ks], fxb[ks], sacc[1]);
+                        sacc[2] = M::mma(fy2[ks], fxb[ks], sacc[2]);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             } else {
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks)
-                    sacc[0] = M::mma(*reinterpret_cast<const V8*>(y0 + 32 * ks),
-                                     *reinterpret_cast<const V8*>(xa + 32 * ks), sacc[0]);
+                for (int k0 = 0; k0 < KS; k0 += SB) {
+                    V8 fxa[SB], fy0[SB];
+#pragma unroll
+                    for (int ks = 0; ks < SB; ++ks) {
+                        fxa[ks] = *reinterpret_cast<const V8*>(xa + 32 * (k0 + ks));
+                        fy0[ks] = *reinterpret_cast<const V8*>(y0 + 32 * (k0 + ks));
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int ks = 0; ks < SB; ++ks) sacc[0] = M::mma(fy0[ks], fxa[ks], sacc[0]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
             {
                 V4 p;
@@ -313,14 +355,25 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
             f32x4 oacc[4];
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) oacc[i4] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            constexpr int IB = KS <= 4 ? KS : 2;  // contraction steps per batch of reads
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
+            for (int k0 = 0; k0 < KS; k0 += IB) {
+                V8 bx[IB][4];
 #pragma unroll
-                for (int i4 = 0; i4 < 4; ++i4) {
-                    const T* px = Xs + (16 * i4 + r) * XS + 32 * ks + 4 * g;
-                    const V8 bx = cat<V8, V4>(*reinterpret_cast<const V4*>(px), *reinterpret_cast<const V4*>(px + 16));
-                    oacc[i4] = M::mma(sb[ks], bx, oacc[i4]);
+                for (int ks = 0; ks < IB; ++ks) {
+#pragma unroll
+                    for (int i4 = 0; i4 < 4; ++i4) {
+                        const T* px = Xs + (16 * i4 + r) * XS + 32 * (k0 + ks) + 4 * g;
+                        bx[ks][i4] = cat<V8, V4>(*reinterpret_cast<const V4*>(px), *reinterpret_cast<const V4*>(px + 16));
+                    }
                 }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int ks = 0; ks < IB; ++ks) {
+#pragma unroll
+                    for (int i4 = 0; i4 < 4; ++i4) oacc[i4] = M::mma(sb[k0 + ks], bx[ks][i4], oacc[i4]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
@@ -346,15 +399,22 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
                 f32x4 oacc[4];
 #pragma unroll
                 for (int i4 = 0; i4 < 4; ++i4) oacc[i4] = Ob[(w * 4 + i4) * 64 + lane];
+                V8 bp[4][2];
 #pragma unroll
                 for (int i4 = 0; i4 < 4; ++i4) {
 #pragma unroll
                     for (int ks = 0; ks < 2; ++ks) {
                         const bool need = REVERSE ? (ks >= i4 / 2) : (ks <= i4 / 2);
-                        if (need) {
-                            const V8 bp = *reinterpret_cast<const V8*>(Ps + (16 * i4 + r) * ZS + 32 * ks + 8 * g);
-                            oacc[i4] = M::mma(zf[ks], bp, oacc[i4]);
-                        }
+                        if (need) bp[i4][ks] = *reinterpret_cast<const V8*>(Ps + (16 * i4 + r) * ZS + 32 * ks + 8 * g);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) {
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks) {
+                        const bool need = REVERSE ? (ks >= i4 / 2) : (ks <= i4 / 2);
+                        if (need) oacc[i4] = M::mma(zf[ks], bp[i4][ks], oacc[i4]);
                     }
                 }
                 const int col = col0 + 16 * w + 4 * g;
@@ -376,36 +436,61 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
                 const T* pz = Zs + (32 * ks + 8 * g + (r >> 2)) * ZS + 16 * w + 4 * (r & 3);
                 zf[ks] = cat<V8, V4>(lds_tr4<V4>(pz), lds_tr4<V4>(pz + 4 * ZS));
             }
-            if (DECAY) {
+            constexpr int UB = KT <= 8 ? KT : 4;  // state tiles per batch of transposed reads
 #pragma unroll
-                for (int ks = 0; ks < 2; ++ks)
+            for (int t0 = 0; t0 < KT; t0 += UB) {
+                V8 ay[UB][2];
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) zf[ks][u] = (T)((float)zf[ks][u] * zfac[ks][u]);
+                for (int kt = 0; kt < UB; ++kt) {
 #pragma unroll
-                for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) st[kt][v] *= lamB;
-            }
-#pragma unroll
-            for (int kt = 0; kt < KT; ++kt) {
-#pragma unroll
-                for (int ks = 0; ks < 2; ++ks) {
-                    const T* py = Ys + (32 * ks + 8 * g + (r >> 2)) * XS + 16 * kt + 4 * (r & 3);
-                    const V8 ay = cat<V8, V4>(lds_tr4<V4>(py), lds_tr4<V4>(py + 4 * XS));
-                    st[kt] = M::mma(ay, zf[ks], st[kt]);
+                    for (int ks = 0; ks < 2; ++ks) {
+                        const T* py = Ys + (32 * ks + 8 * g + (r >> 2)) * XS + 16 * (t0 + kt) + 4 * (r & 3);
+                        ay[kt][ks] = cat<V8, V4>(lds_tr4<V4>(py), lds_tr4<V4>(py + 4 * XS));
+                    }
                 }
+                __builtin_amdgcn_sched_barrier(0);
+                if (DECAY && t0 == 0) {
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) zf[ks][u] = (T)((float)zf[ks][u] * zfac[ks][u]);
+#pragma unroll
+                    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) st[kt][v] *= lamB;
+                }
+#pragma unroll
+                for (int kt = 0; kt < UB; ++kt) {
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks) st[t0 + kt] = M::mma(ay[kt][ks], zf[ks], st[t0 + kt]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-        if (NBUF == 2) {
-            if (have_next) stage_block((int)((it + 1) & 1));
+        if (NSET == 2) {
+            __syncthreads();
+        } else if (NBUF == 2) {
+            stage_block((int)((it + 1) & 1), xr, yr, zr);
+            load_block(it + 2, xr, yr, zr);
             __syncthreads();
         } else {
             __syncthreads();
-            if (have_next) {
-                stage_block(0);
-                __syncthreads();
-            }
+            stage_block(0, xr, yr, zr);
+            load_block(it + 2, xr, yr, zr);
+            __syncthreads();
         }
+    };
+    if (NSET == 2) {
+        // Both halves of the unrolled loop always run, so the two register sets are refilled in the
+        // same order on every path and the wait before staging one set leaves the other in flight.
+        int64_t it = 0;
+        for (; it + 1 < it_end; it += 2) {
+            block_body(it, xrB, yrB, zrB);
+            block_body(it + 1, xrA, yrA, zrA);
+        }
+        if (it < it_end) block_body(it, xrB, yrB, zrB);
+    } else {
+        for (int64_t it = 0; it < it_end; ++it) block_body(it, xrA, yrA, zrA);
     }
 }
 
