@@ -1,0 +1,75 @@
+// Definitions shared by the sweep kernels (bf16 / fp16 MFMA paths).
+#pragma once
+#include "la_common.h"
+
+namespace la {
+
+struct SweepArgs {
+    const void* x;  // (bh, n, dk)
+    const void* y;  // (bh, n, dk)
+    const void* z;  // (bh, n, dv)
+    void* out;      // (bh, n, dv)
+    const float* s; // h decay rates or nullptr
+    int64_t n;
+    int dk, dv, h, bh, nslice;
+    int nchunk;          // sequence chunks per (batch, head, slice); 1 = one workgroup walks the whole sequence
+    int chunk_start[9];  // first 64-token block (in walk order) of each chunk; chunk_start[nchunk] = number of blocks
+};
+
+template <typename T>
+struct Mma;
+template <>
+struct Mma<__bf16> {
+    typedef bf16x8 V8;
+    typedef bf16x4 V4;
+    static __device__ __forceinline__ f32x4 mma(V8 a, V8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ __bf16 cvt(float f) { return (__bf16)f; }
+};
+template <>
+struct Mma<_Float16> {
+    typedef f16x8 V8;
+    typedef f16x4 V4;
+    static __device__ __forceinline__ f32x4 mma(V8 a, V8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+    // fp16 saturates instead of overflowing to inf when a state entry is large
+    static __device__ __forceinline__ _Float16 cvt(float f) {
+        return (_Float16)__builtin_fminf(__builtin_fmaxf(f, -65504.f), 65504.f);
+    }
+};
+
+// LDS transpose read: the 16 lanes of a group each point at 4 consecutive
+// 16-bit elements; lane i of the group receives element (i % 4) of the lanes
+// 4e + i/4, e = 0..3.  With lane L pointing at row L/4, columns 4(L%4).. of a
+// row-major tile, lane i ends up with column i of rows 0..3.
+template <typename V4>
+__device__ __forceinline__ V4 lds_tr4(const void* p) {
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p));
+    return __builtin_bit_cast(V4, v);
+}
+template <typename V8, typename V4>
+__device__ __forceinline__ V8 cat(V4 a, V4 b) {
+    return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// The 10 non-masked 16x16 tiles of the 64x64 score block, dealt to the four score
+// waves: slot 0 is tile (jt0, itA), slots 1,2 are (jt1, itB), (jt2, itB); -1 = none.
+// Written for the forward direction (jt <= it); the reverse direction mirrors
+// both indices (3 - jt, 3 - it).
+struct TileDeal {
+    int itA, jt0, itB, jt1, jt2;
+};
+__device__ __constant__ const TileDeal kDeal[4] = {
+    {3, 0, 3, 1, 2},
+    {3, 3, 2, 0, 1},
+    {2, 2, 1, 0, 1},
+    {0, 0, -1, -1, -1},
+};
+
+// Launches the single-barrier pipelined kernel (feature dim up to 128); defined in la_sweep_pipe.hip.
+int sweep_pipe(const SweepArgs& a, int dtype, bool reverse, hipStream_t st);
+
+}  // namespace la

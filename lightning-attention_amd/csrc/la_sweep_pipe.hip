@@ -1,0 +1,455 @@
+// Single-sweep decayed linear attention for gfx950, feature dim up to 128:
+// software-pipelined variant with one workgroup barrier per 64-token block.
+//
+// Same operator and the same division of the data as la_sweep.hip (one workgroup of
+// 8 wavefronts per (batch, head, 64-column slice of z/out), 64-token blocks walked in
+// order, fp32 state in MFMA accumulators), but the two kinds of wavefronts work on
+// different blocks at the same time:
+//   waves 0-3 ("score" waves)  during iteration `it` they compute the masked, decayed
+//                              score tile P of block it+1 and leave it in LDS;
+//   waves 4-7 ("state" waves)  own a dk x 16 column slab of the state and finish block
+//                              `it`: out^T = Lout * (state^T x^T) + z^T P^T, store, then
+//                              state = lam^64 state + y^T (z * Lupd).
+// The inter-block term therefore never leaves registers, nothing is handed from one kind of
+// wave to the other inside an iteration, and a single barrier per iteration orders
+//   - the x/y/z tiles: three LDS buffers (block `it` read by the state waves, block it+1
+//     read by the score waves, block it+2 being written), fed from two register sets so that
+//     blocks it+3 and it+4 are in flight from memory;
+//   - the P tiles: two LDS buffers (block `it` read, block it+1 written).
+// (lightning_attn/ops/triton/lightning_attn2.py:8-85 forward, :88-395 backward.)
+#include "la_sweep_common.h"
+#include "lightning_attn_hip.h"
+
+namespace la {
+
+template <int DKP>
+struct PipeLds {
+#ifndef LA_PIPE_XPAD
+#define LA_PIPE_XPAD 16
+#endif
+    static constexpr int XS = DKP + LA_PIPE_XPAD;  // row stride (elements) of the x / y tiles
+#ifndef LA_PIPE_PPAD
+#define LA_PIPE_PPAD 8
+#endif
+    static constexpr int ZS = 64 + 8;             // row stride of the z slice
+    static constexpr int PS = 64 + LA_PIPE_PPAD;  // row stride of the P tile
+    static constexpr int XY = 2 * 64 * XS;        // elements of one x + y buffer
+    static constexpr int ZT = 64 * ZS;            // elements of one z buffer
+    static constexpr int PT = 64 * PS;            // elements of one P buffer
+    static constexpr size_t bytes(size_t elt) { return (size_t)(3 * XY + 3 * ZT + 2 * PT) * elt; }
+};
+
+template <typename T, int DKP, bool REVERSE, bool DECAY>
+__global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepArgs a) {
+    typedef Mma<T> M;
+    typedef typename M::V8 V8;
+    typedef typename M::V4 V4;
+    typedef PipeLds<DKP> L;
+    constexpr int XS = L::XS, ZS = L::ZS, PS = L::PS;
+    constexpr int KS = DKP / 32;  // 32-wide contraction steps over the feature dim
+    constexpr int KT = DKP / 16;  // 16-row state tiles
+    constexpr int XC = DKP / 64;  // 16-byte chunks per thread for an x / y tile (512 threads)
+    extern __shared__ __align__(16) unsigned char smem[];
+    // LDS map in bytes: [3][x 64*XS | y 64*XS] tiles, [3][64*ZS] z tiles, [2][64*PS] P tiles.
+    // All LDS accesses below are written as (per-iteration base register) + (compile-time
+    // constant), which the DS instructions take as register + immediate offset; the bases are
+    // made opaque to the optimiser once per iteration so that it does not keep one address
+    // register per access alive across the loop.
+    constexpr unsigned E = (unsigned)sizeof(T);
+    constexpr unsigned XYB = L::XY * E, ZTB = L::ZT * E, PTB = L::PT * E, YOFF = 64 * XS * E;
+    constexpr unsigned ZBASE = 3 * XYB, PBASE = ZBASE + 3 * ZTB;
+    auto opaque = [](unsigned v) {
+        asm volatile("" : "+v"(v));
+        return v;
+    };
+    auto ld8 = [&](unsigned addr) { return *reinterpret_cast<const V8*>(smem + addr); };
+    auto ld4 = [&](unsigned addr) { return *reinterpret_cast<const V4*>(smem + addr); };
+    auto ldt = [&](unsigned addr) { return lds_tr4<V4>(smem + addr); };
+
+    // Workgroups are dealt round-robin to the 8 XCDs by linear id; keep the
+    // column slices of one head on one XCD so their x / y re-reads share an L2.
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int per_unit = a.nslice * a.nchunk;
+    const int unit = xcd + 8 * (local / per_unit);
+    const int slice = (local % per_unit) % a.nslice;
+    const int chunk = (local % per_unit) / a.nslice;
+    if (unit >= a.bh) return;
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool state_role = wave >= 4;
+    const int w = wave & 3;
+    const int lane = tid & 63, r = lane & 15, g = lane >> 4;
+    const int64_t n = a.n;
+    const int dk = a.dk, dv = a.dv;
+    // one bounds-checked buffer per (batch, head) slice: rows >= n read as zero / are not written
+    const __amdgpu_buffer_rsrc_t xb = make_rsrc(static_cast<const T*>(a.x) + (int64_t)unit * n * dk, (unsigned)(n * dk * sizeof(T)));
+    const __amdgpu_buffer_rsrc_t yb = make_rsrc(static_cast<const T*>(a.y) + (int64_t)unit * n * dk, (unsigned)(n * dk * sizeof(T)));
+    const __amdgpu_buffer_rsrc_t zb = make_rsrc(static_cast<const T*>(a.z) + (int64_t)unit * n * dv, (unsigned)(n * dv * sizeof(T)));
+    const __amdgpu_buffer_rsrc_t ob = make_rsrc(static_cast<T*>(a.out) + (int64_t)unit * n * dv, (unsigned)(n * dv * sizeof(T)));
+    const int col0 = slice * 64;
+    const bool cols_active = (col0 + 16 * w) < dv;
+
+    float rate = 0.f;
+    if (DECAY) rate = a.s[unit % a.h];
+
+    // ---- score waves: the tiles of this wave ------------------------------------
+    TileDeal deal = kDeal[w];
+    if (REVERSE) {
+        deal.itA = 3 - deal.itA; deal.jt0 = 3 - deal.jt0;
+        if (deal.itB >= 0) { deal.itB = 3 - deal.itB; deal.jt1 = 3 - deal.jt1; deal.jt2 = 3 - deal.jt2; }
+    }
+    const int itA = __builtin_amdgcn_readfirstlane(deal.itA), jt0 = __builtin_amdgcn_readfirstlane(deal.jt0);
+    const int itB = __builtin_amdgcn_readfirstlane(deal.itB), jt1 = __builtin_amdgcn_readfirstlane(deal.jt1);
+    const int jt2 = __builtin_amdgcn_readfirstlane(deal.jt2);
+    // Per-lane constant factors (all <= 1); the two kinds of waves keep theirs in the same registers.
+    //   score waves: cf[4 sl + v]  mask * decay of element v of score tile slot sl
+    //   state waves: cf[it]        scale of the inter-block term for token i = 16 it + r
+    //                cf[4 + 8 ks + u]  scale of token j = 32 ks + 8 g + u in the state update
+    float cf[20];
+#pragma unroll
+    for (int i = 0; i < 20; ++i) cf[i] = 1.f;
+    float lamB = 1.f;
+    if (!state_role) {
+        const int its[3] = {itA, itB, itB}, jts[3] = {jt0, jt1, jt2};
+#pragma unroll
+        for (int sl = 0; sl < 3; ++sl)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int i = 16 * its[sl] + r, j = 16 * jts[sl] + 4 * g + v;
+                const int diff = REVERSE ? (j - i) : (i - j);
+                cf[4 * sl + v] = diff >= 0 ? (DECAY ? expf(-rate * (float)diff) : 1.f) : 0.f;
+            }
+    } else if (DECAY) {
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int i = 16 * it + r;
+            cf[it] = expf(-rate * (float)(REVERSE ? 64 - i : i));
+        }
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int j = 32 * ks + 8 * g + u;
+                cf[4 + 8 * ks + u] = expf(-rate * (float)(REVERSE ? j : 64 - j));
+            }
+        lamB = expf(-rate * 64.f);
+    }
+
+    f32x4 st[KT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) st[kt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    const int64_t nblk = (n + 63) / 64;
+    // Sequence chunking: this workgroup produces the blocks [it_first, it_end) of the walk.  It
+    // first runs over the blocks before it_first with the state update only ("warm-up": y and z
+    // are read, nothing is written) to rebuild the state its chunk starts from.
+    const int64_t it_first = a.chunk_start[chunk];
+    const int64_t it_end = a.chunk_start[chunk + 1];
+
+    u32x4 xrA[XC], yrA[XC], zrA, xrB[XC], yrB[XC], zrB;
+
+    // Fetches block number b of the walk.  Blocks at or beyond it_end, and the x tile of warm-up
+    // blocks, are fetched at the out-of-range offset: zeros, no memory traffic, and the sequence of
+    // memory operations is the same for every wave on every path (the waits the compiler places
+    // before the staging can then leave the younger operations in flight).
+    auto load_block = [&](int64_t b, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4& zr) {
+        const int64_t t = REVERSE ? nblk - 1 - b : b;
+        const bool valid = b < it_end, need_x = valid && b >= it_first;
+        const unsigned tok0 = (unsigned)(t * 64);
+#pragma unroll
+        for (int u = 0; u < XC; ++u) {
+            const int c = tid + 512 * u;
+            const int row = c / (DKP / 8), col = (c % (DKP / 8)) * 8;
+            // columns dk..DKP-1 are zero padding
+            const unsigned off = col < dk ? ((tok0 + row) * (unsigned)dk + col) * (unsigned)sizeof(T) : kOob;
+            xr[u] = buf_load16(xb, need_x ? off : kOob);
+            yr[u] = buf_load16(yb, valid ? off : kOob);
+        }
+        {
+            const int row = tid / 8, col = (tid % 8) * 8;
+            const unsigned off = (col0 + col < dv) ? ((tok0 + row) * (unsigned)dv + col0 + col) * (unsigned)sizeof(T) : kOob;
+            zr = buf_load16(zb, valid ? off : kOob);
+        }
+    };
+    const unsigned lane_stage_xy = ((tid / (DKP / 8)) * XS + (tid % (DKP / 8)) * 8) * E;
+    const unsigned lane_stage_z = ((tid / 8) * ZS + (tid % 8) * 8) * E;
+    auto stage_block = [&](int buf, const u32x4 (&xr)[XC], const u32x4 (&yr)[XC], const u32x4& zr) {
+        const unsigned xd = opaque(buf * XYB + lane_stage_xy);
+        const unsigned zd = opaque(ZBASE + buf * ZTB + lane_stage_z);
+#pragma unroll
+        for (int u = 0; u < XC; ++u) {
+            // chunk c = tid + 512 u lies (512 / (DKP / 8)) rows below chunk tid
+            constexpr unsigned ROWS = 512 / (DKP / 8);
+            *reinterpret_cast<u32x4*>(smem + xd + u * ROWS * XS * E) = xr[u];
+            *reinterpret_cast<u32x4*>(smem + xd + YOFF + u * ROWS * XS * E) = yr[u];
+        }
+        *reinterpret_cast<u32x4*>(smem + zd) = zr;
+    };
+
+    // Score waves: S^T tiles of this wave for the block in tile buffer `buf` -> masked, decayed
+    // P[i][j] in P buffer `pbuf`.  All fragment reads are issued before the MFMAs (the scheduler
+    // otherwise sinks each read next to its use and the wave pays one LDS round trip per MFMA).
+    const unsigned lane_frag = (r * XS + 8 * g) * E;   // row r, 16-byte chunk g of an x / y tile
+    const unsigned lane_pw = (r * PS + 4 * g) * E;     // P[i = r][j = 4g ..] within a 16 x 16 tile
+    auto score_block = [&](int buf, int pbuf) {
+        const unsigned xbase = buf * XYB + lane_frag, pbase = PBASE + pbuf * PTB + lane_pw;
+        f32x4 sacc[3];
+#pragma unroll
+        for (int sl = 0; sl < 3; ++sl) sacc[sl] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        const unsigned xa = opaque(xbase + 16 * itA * XS * E);
+        const unsigned y0 = opaque(xbase + YOFF + 16 * jt0 * XS * E);
+        if (itB >= 0) {
+            const unsigned xb2 = opaque(xbase + 16 * itB * XS * E);
+            const unsigned y1 = opaque(xbase + YOFF + 16 * jt1 * XS * E);
+            const unsigned y2 = opaque(xbase + YOFF + 16 * jt2 * XS * E);
+            V8 fxa[KS], fxb[KS], fy0[KS], fy1[KS], fy2[KS];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                fxa[ks] = ld8(xa + 32 * ks * E);
+                fy0[ks] = ld8(y0 + 32 * ks * E);
+                fxb[ks] = ld8(xb2 + 32 * ks * E);
+                fy1[ks] = ld8(y1 + 32 * ks * E);
+                fy2[ks] = ld8(y2 + 32 * ks * E);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                sacc[0] = M::mma(fy0[ks], fxa[ks], sacc[0]);
+                sacc[1] = M::mma(fy1[ks], fxb[ks], sacc[1]);
+                sacc[2] = M::mma(fy2[ks], fxb[ks], sacc[2]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        } else {
+            V8 fxa[KS], fy0[KS];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                fxa[ks] = ld8(xa + 32 * ks * E);
+                fy0[ks] = ld8(y0 + 32 * ks * E);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) sacc[0] = M::mma(fy0[ks], fxa[ks], sacc[0]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        {
+            V4 p;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[0][v] * cf[v]);
+            *reinterpret_cast<V4*>(smem + opaque(pbase + (16 * itA * PS + 16 * jt0) * E)) = p;
+        }
+        if (itB >= 0) {
+            V4 p;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[1][v] * cf[4 + v]);
+            *reinterpret_cast<V4*>(smem + opaque(pbase + (16 * itB * PS + 16 * jt1) * E)) = p;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[2][v] * cf[8 + v]);
+            *reinterpret_cast<V4*>(smem + opaque(pbase + (16 * itB * PS + 16 * jt2) * E)) = p;
+        }
+    };
+
+    // zero both P buffers once: tiles on the masked side of the diagonal are never written
+    for (int c = tid; c < 2 * L::PT / 8; c += 512) reinterpret_cast<uint4*>(smem + PBASE)[c] = make_uint4(0, 0, 0, 0);
+    load_block(0, xrA, yrA, zrA);
+    load_block(1, xrB, yrB, zrB);
+    stage_block(0, xrA, yrA, zrA);
+    load_block(2, xrA, yrA, zrA);
+    stage_block(1, xrB, yrB, zrB);
+    load_block(3, xrB, yrB, zrB);
+    __syncthreads();
+    if (!state_role && it_first == 0) score_block(0, 0);
+    __syncthreads();
+
+    // state-wave lane offsets: x fragment halves (row r, columns 4g..), transposed reads of y and
+    // of this wave's 16 z columns (row 8g + r/4, columns 4 (r%4)..), P fragments (row r, chunk g)
+    const unsigned lane_xq = (r * XS + 4 * g) * E;
+    const unsigned lane_yt = ((8 * g + (r >> 2)) * XS + 4 * (r & 3)) * E;
+    const unsigned lane_zt = ((8 * g + (r >> 2)) * ZS + 16 * w + 4 * (r & 3)) * E;
+    const unsigned lane_pr = (r * PS + 8 * g) * E;
+
+    // One iteration.  `xr, yr, zr` hold block it+2 on entry and block it+4 on exit.
+    auto iteration = [&](const int64_t it, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4& zr) {
+        const int64_t t = REVERSE ? nblk - 1 - it : it;
+        const bool have_next = it + 1 < it_end;
+        const bool warm = it < it_first;  // warm-up block: state update only
+        const int bcur = (int)((unsigned)it % 3u);
+        const int bnext = bcur == 2 ? 0 : bcur + 1;
+        const int bstage = bnext == 2 ? 0 : bnext + 1;
+        // publish block it+2 (its buffer was last read in iteration it-1) and refill the
+        // registers with block it+4
+        stage_block(bstage, xr, yr, zr);
+        load_block(it + 4, xr, yr, zr);
+
+        // Every wave issues four stores per iteration; where it has nothing to write they go to the
+        // out-of-range offset and the hardware drops them.  All waves then run the same sequence of
+        // memory operations on every path.
+        auto dummy_stores = [&]() {
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) buf_store8(ob, kOob, (u32x2){0u, 0u});
+        };
+        if (!state_role) {
+            if (have_next && it + 1 >= it_first) score_block(bnext, (int)((it + 1) & 1));
+            dummy_stores();
+        } else if (cols_active) {
+            const unsigned xq = opaque(bcur * XYB + lane_xq);
+            const unsigned yq = opaque(bcur * XYB + YOFF + lane_yt);
+            const unsigned zq = opaque(ZBASE + bcur * ZTB + lane_zt);
+            const unsigned pq = opaque(PBASE + (unsigned)(it & 1) * PTB + lane_pr);
+            // z^T fragments of this wave's 16 columns: A operand of the intra-block product and,
+            // scaled, B operand of the state update
+            V8 zf[2];
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                zf[ks] = cat<V8, V4>(ldt(zq + 32 * ks * ZS * E), ldt(zq + (32 * ks + 4) * ZS * E));
+            }
+            if (!warm) {
+                // out^T[c][i] = Lout[i] * sum_k state[k][c] x[i][k]  +  sum_j z[j][c] P[i][j]
+                // The x fragments of contraction step ks+1 (and, at the end, the P fragments) are
+                // read while the MFMAs of step ks run.
+                auto read_x = [&](int ks, V8 (&bx)[4]) {
+#pragma unroll
+                    for (int i4 = 0; i4 < 4; ++i4) {
+                        // 8-byte reads from unrelated base registers (one per contraction step and
+                        // half): fused in pairs into ds_read2_b64 they would conflict on the LDS
+                        // banks at this row stride
+                        const unsigned lo = opaque(xq + 32 * ks * E), hi = opaque(xq + (32 * ks + 16) * E);
+                        bx[i4] = cat<V8, V4>(ld4(lo + 16 * i4 * XS * E), ld4(hi + 16 * i4 * XS * E));
+                    }
+                };
+                V8 bx[2][4];
+                V8 bp[4][2];
+                read_x(0, bx[0]);
+                f32x4 oacc[4];
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) oacc[i4] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    if (ks + 1 < KS) {
+                        read_x(ks + 1, bx[(ks + 1) & 1]);
+                    } else {
+#pragma unroll
+                        for (int i4 = 0; i4 < 4; ++i4) {
+#pragma unroll
+                            for (int k2 = 0; k2 < 2; ++k2) {
+                                const bool need = REVERSE ? (k2 >= i4 / 2) : (k2 <= i4 / 2);
+                                if (need) bp[i4][k2] = ld8(pq + (16 * i4 * PS + 32 * k2) * E);
+                            }
+                        }
+                    }
+                    V8 sb;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        sb[v] = M::cvt(st[2 * ks][v]);
+                        sb[4 + v] = M::cvt(st[2 * ks + 1][v]);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int i4 = 0; i4 < 4; ++i4) oacc[i4] = M::mma(sb, bx[ks & 1][i4], oacc[i4]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if (DECAY) {
+#pragma unroll
+                    for (int i4 = 0; i4 < 4; ++i4)
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) oacc[i4][v] *= cf[i4];
+                }
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) {
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks) {
+                        const bool need = REVERSE ? (ks >= i4 / 2) : (ks <= i4 / 2);
+                        if (need) oacc[i4] = M::mma(zf[ks], bp[i4][ks], oacc[i4]);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                const int col = col0 + 16 * w + 4 * g;
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) {
+                    const unsigned tok = (unsigned)(t * 64) + 16 * i4 + r;
+                    V4 o;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) o[v] = (T)oacc[i4][v];
+                    const unsigned off = col < dv ? (tok * (unsigned)dv + col) * (unsigned)sizeof(T) : kOob;
+                    buf_store8(ob, off, __builtin_bit_cast(u32x2, o));
+                }
+            } else {
+                dummy_stores();
+            }
+            if (have_next) {
+                // state = lam^64 state + y^T (z * Lupd)
+                V8 ay[KT][2];
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks) {
+                        const unsigned py = yq + (32 * ks * XS + 16 * kt) * E;
+                        ay[kt][ks] = cat<V8, V4>(ldt(py), ldt(py + 4 * XS * E));
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if (DECAY) {
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) zf[ks][u] = (T)((float)zf[ks][u] * cf[4 + 8 * ks + u]);
+#pragma unroll
+                    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) st[kt][v] *= lamB;
+                }
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks) st[kt] = M::mma(ay[kt][ks], zf[ks], st[kt]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+            dummy_stores();
+        }
+        __syncthreads();
+    };
+    // Both halves of the unrolled loop always run, so the two register sets are refilled in the
+    // same order on every path and the wait before staging one set leaves the other in flight.
+    int64_t it = 0;
+    for (; it + 1 < it_end; it += 2) {
+        iteration(it, xrA, yrA, zrA);
+        iteration(it + 1, xrB, yrB, zrB);
+    }
+    if (it < it_end) iteration(it, xrA, yrA, zrA);
+}
+
+template <typename T, int DKP, bool REVERSE, bool DECAY>
+static int launch_one(const SweepArgs& a, hipStream_t st) {
+    constexpr size_t lds = PipeLds<DKP>::bytes(sizeof(T));
+    static_assert(lds <= 160 * 1024, "LDS budget");
+    auto kern = la_sweep_pipe_kernel<T, DKP, REVERSE, DECAY>;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+    }
+    const int units8 = (a.bh + 7) / 8 * 8;
+    const unsigned grid = (unsigned)(units8 * a.nslice * a.nchunk);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, st, a);
+    return (int)hipGetLastError();
+}
+
+template <typename T, bool REVERSE>
+static int launch_dir(const SweepArgs& a, hipStream_t st) {
+    const bool decay = a.s != nullptr;
+#define LA_GO(DKP) (decay ? launch_one<T, DKP, REVERSE, true>(a, st) : launch_one<T, DKP, REVERSE, false>(a, st))
+    if (a.dk <= 64) return LA_GO(64);
+    return LA_GO(128);
+#undef LA_GO
+}
+
+int sweep_pipe(const SweepArgs& a, int dtype, bool reverse, hipStream_t st) {
+    if (a.dk > 128) return LA_E_UNSUPPORTED;
+    if (dtype == LA_BF16) return reverse ? launch_dir<__bf16, true>(a, st) : launch_dir<__bf16, false>(a, st);
+    if (dtype == LA_FP16) return reverse ? launch_dir<_Float16, true>(a, st) : launch_dir<_Float16, false>(a, st);
+    return LA_E_UNSUPPORTED;
+}
+
+}  // namespace la
