@@ -33,7 +33,7 @@ namespace la {
 template <int DKP>
 struct SweepLds {
 #ifndef LA_XPAD
-#define LA_XPAD 8
+#define LA_XPAD 16
 #endif
 #ifndef LA_ZPAD
 #define LA_ZPAD 8
@@ -298,8 +298,15 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
                 for (int ks = 0; ks < IB; ++ks) {
 #pragma unroll
                     for (int i4 = 0; i4 < 4; ++i4) {
-                        const T* px = Xs + (16 * i4 + r) * XS + 32 * (k0 + ks) + 4 * g;
-                        bx[ks][i4] = cat<V8, V4>(*reinterpret_cast<const V4*>(px), *reinterpret_cast<const V4*>(px + 16));
+                        // two 8-byte reads from base registers the optimiser cannot relate: fused
+                        // into one ds_read2_b64 they would conflict on the LDS banks
+                        const unsigned xoff = (unsigned)((buf * L::TILE + r * XS + 32 * (k0 + ks) + 4 * g) * sizeof(T));
+                        unsigned lo = xoff, hi = xoff + 16 * (unsigned)sizeof(T);
+                        asm volatile("" : "+v"(lo));
+                        asm volatile("" : "+v"(hi));
+                        constexpr unsigned ROW = 16 * XS * (unsigned)sizeof(T);
+                        bx[ks][i4] = cat<V8, V4>(*reinterpret_cast<const V4*>(smem + lo + i4 * ROW),
+                                                 *reinterpret_cast<const V4*>(smem + hi + i4 * ROW));
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -449,8 +456,6 @@ template <typename T, bool REVERSE>
 static int launch_dir(const SweepArgs& a, hipStream_t st) {
     const bool decay = a.s != nullptr;
 #define LA_GO(DKP) (decay ? launch_one<T, DKP, REVERSE, true>(a, st) : launch_one<T, DKP, REVERSE, false>(a, st))
-    if (a.dk <= 64) return LA_GO(64);
-    if (a.dk <= 128) return LA_GO(128);
     if (a.dk <= 192) return LA_GO(192);
     return LA_GO(256);
 #undef LA_GO
@@ -508,10 +513,7 @@ int sweep(const void* x, const void* y, const void* z, void* out, const float* s
     a.n = n; a.dk = (int)dk; a.dv = (int)dv; a.h = (int)h; a.bh = (int)bh;
     a.nslice = (int)((dv + 63) / 64);
     choose_chunks(a);
-    if (dk <= 128) {
-        const char* env = getenv("LA_SWEEP_PIPE");
-        if (!(env && env[0] == '0')) return sweep_pipe(a, dtype, reverse, st);
-    }
+    if (dk <= 128) return sweep_pipe(a, dtype, reverse, st);  // pipelined kernel, la_sweep_pipe.hip
     if (dtype == LA_BF16) return reverse ? launch_dir<__bf16, true>(a, st) : launch_dir<__bf16, false>(a, st);
     if (dtype == LA_FP16) return reverse ? launch_dir<_Float16, true>(a, st) : launch_dir<_Float16, false>(a, st);
     return LA_E_UNSUPPORTED;
