@@ -77,6 +77,28 @@ int la_bwd(const void *q, const void *k, const void *v, const float *s, const vo
            void *workspace, size_t ws_bytes, void *stream);
 
 /*
+ * la_fwd / la_bwd on tensors that are not plain (b,h,n,d) arrays: every tensor argument gets
+ * three strides in ELEMENTS (batch, head, token), in the order of the pointer arguments
+ * (la_fwd_strided: q,k,v,o = 12 values; la_bwd_strided: q,k,v,dout,dq,dk,dv = 21 values); the
+ * feature dim stays contiguous.  A projection output (b,n,h*d) is then used in place with
+ * strides {n*h*d, d, h*d}, and o / dq / dk / dv can be written in that layout too.  This removes
+ * the copies the reference makes around the operator: `.contiguous()` on q,k,v,do
+ * (lightning_attn/ops/triton/lightning_attn2.py:402-405, 439-442) after the caller's
+ * `rearrange(x, "b n (h d) -> b h n d")` and the copy behind `rearrange(o, "b h n d -> b n (h d)")`
+ * (examples/module/tnl_attn.py:56-64).  Strides must be multiples of 16 bytes, token stride >=
+ * the feature dim, one (batch, head) sequence below 2 GiB; bf16 / fp16 only (float32 tensors must
+ * be plain: LA_E_UNSUPPORTED otherwise).
+ */
+int la_fwd_strided(const void *q, const void *k, const void *v, const float *s, void *o,
+                   const int64_t *strides,
+                   int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
+                   void *workspace, size_t ws_bytes, void *stream);
+int la_bwd_strided(const void *q, const void *k, const void *v, const float *s, const void *dout,
+                   void *dq, void *dk, void *dv, const int64_t *strides,
+                   int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
+                   void *workspace, size_t ws_bytes, void *stream);
+
+/*
  * SimpleRMSNorm forward: rstd[r] = 1/sqrt(mean(x[r,:]^2) + eps), y = x * rstd.
  * x,y: rows x cols with `row_stride` elements between rows; rstd: rows floats.
  * Replaces _SrmsNorm.forward + srms_norm_fw

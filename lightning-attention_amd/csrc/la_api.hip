@@ -1,18 +1,35 @@
 // extern "C" entry points of the attention path (see include/lightning_attn_hip.h).
-#include "la_common.h"
+#include "la_sweep_common.h"
 #include "lightning_attn_hip.h"
 
 namespace la {
-int sweep(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h, int64_t n,
-          int64_t dk, int64_t dv, int dtype, bool reverse, hipStream_t st);
+int sweep(const void* x, const void* y, const void* z, void* out, const Layout& lx, const Layout& ly, const Layout& lz,
+          const Layout& lo, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
+          bool reverse, hipStream_t st);
 int sweep_f32(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
               int64_t n, int64_t dk, int64_t dv, bool reverse, hipStream_t st);
 
+// A tensor argument: device pointer + where its (batch, head, token) rows start.
+struct Tensor {
+    const void* p;
+    Layout l;
+};
+static Tensor dense(const void* p, int64_t h, int64_t n, int64_t cols) { return Tensor{p, Layout{h * n * cols, n * cols, cols}}; }
+static Tensor strided(const void* p, const int64_t* st) { return Tensor{p, Layout{st[0], st[1], st[2]}}; }
+static bool is_dense(const Tensor& t, int64_t h, int64_t n, int64_t cols) {
+    return t.l.ts == cols && t.l.hs == n * cols && t.l.bs == h * n * cols;
+}
+
 // one directional sweep at the element type named by dtype
-static int run(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
+static int run(const Tensor& x, const Tensor& y, const Tensor& z, const Tensor& out, const float* s, int64_t bh, int64_t h,
                int64_t n, int64_t dk, int64_t dv, int dtype, bool reverse, hipStream_t st) {
-    if (dtype == LA_FP32) return sweep_f32(x, y, z, out, s, bh, h, n, dk, dv, reverse, st);
-    return sweep(x, y, z, out, s, bh, h, n, dk, dv, dtype, reverse, st);
+    if (dtype == LA_FP32) {
+        // the float32 accuracy kernel takes plain (b, h, n, d) tensors only
+        if (!is_dense(x, h, n, dk) || !is_dense(y, h, n, dk) || !is_dense(z, h, n, dv) || !is_dense(out, h, n, dv))
+            return LA_E_UNSUPPORTED;
+        return sweep_f32(x.p, y.p, z.p, const_cast<void*>(out.p), s, bh, h, n, dk, dv, reverse, st);
+    }
+    return sweep(x.p, y.p, z.p, const_cast<void*>(out.p), x.l, y.l, z.l, out.l, s, bh, h, n, dk, dv, dtype, reverse, st);
 }
 
 static inline bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -24,6 +41,55 @@ static int check_dims(int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int
     if (n * (d > e ? d : e) * 4 >= (1LL << 31)) return LA_E_SHAPE;
     if (!la_supported(d, e, dtype)) return LA_E_UNSUPPORTED;
     return LA_OK;
+}
+
+// pointer and strides of one tensor with `cols` features per row
+static int check_tensor(const Tensor& t, int64_t b, int64_t h, int64_t n, int64_t cols, int dtype) {
+    if (!t.p) return LA_E_NULLPTR;
+    const int64_t elt = dtype == LA_FP32 ? 4 : 2;
+    if (!al16(t.p) || (t.l.bs * elt) % 16 || (t.l.hs * elt) % 16 || (t.l.ts * elt) % 16) return LA_E_ALIGN;
+    if (t.l.ts < cols || t.l.hs < 0 || t.l.bs < 0) return LA_E_SHAPE;
+    if (b > 1 && t.l.bs == 0) return LA_E_SHAPE;
+    if (h > 1 && t.l.hs == 0) return LA_E_SHAPE;
+    // one (batch, head) sequence is addressed with 32-bit byte offsets below 2 GiB
+    if (((n - 1) * t.l.ts + cols) * elt >= (1LL << 31)) return LA_E_SHAPE;
+    return LA_OK;
+}
+
+static int fwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s, const Tensor& o, int64_t b, int64_t h,
+               int64_t n, int64_t d, int64_t e, int dtype, hipStream_t st) {
+    int rc = check_dims(b, h, n, d, e, dtype);
+    if (rc != LA_OK) return rc;
+    if (b == 0 || n == 0) return LA_OK;  // nothing to do; empty tensors may carry null pointers
+    const Tensor* ts[4] = {&q, &k, &v, &o};
+    const int64_t cols[4] = {d, d, e, e};
+    for (int i = 0; i < 4; ++i)
+        if (!ts[i]->p) return LA_E_NULLPTR;
+    for (int i = 0; i < 4; ++i)
+        if ((rc = check_tensor(*ts[i], b, h, n, cols[i], dtype)) != LA_OK) return rc;
+    return run(q, k, v, o, s, b * h, h, n, d, e, dtype, false, st);
+}
+
+static int bwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s, const Tensor& dout, const Tensor& dq,
+               const Tensor& dk, const Tensor& dv, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
+               hipStream_t st) {
+    int rc = check_dims(b, h, n, d, e, dtype);
+    if (rc != LA_OK) return rc;
+    if (b == 0 || n == 0) return LA_OK;
+    const Tensor* ts[7] = {&q, &k, &v, &dout, &dq, &dk, &dv};
+    const int64_t cols[7] = {d, d, e, e, d, d, e};
+    for (int i = 0; i < 7; ++i)
+        if (!ts[i]->p) return LA_E_NULLPTR;
+    for (int i = 0; i < 7; ++i)
+        if ((rc = check_tensor(*ts[i], b, h, n, cols[i], dtype)) != LA_OK) return rc;
+    // dQ_i = sum_{j<=i} lam^(i-j) (dO_i . v_j) k_j
+    rc = run(dout, v, k, dq, s, b * h, h, n, e, d, dtype, false, st);
+    if (rc != LA_OK) return rc;
+    // dK_j = sum_{i>=j} lam^(i-j) (v_j . dO_i) q_i
+    rc = run(v, dout, q, dk, s, b * h, h, n, e, d, dtype, true, st);
+    if (rc != LA_OK) return rc;
+    // dV_j = sum_{i>=j} lam^(i-j) (k_j . q_i) dO_i
+    return run(k, q, dout, dv, s, b * h, h, n, d, e, dtype, true, st);
 }
 }  // namespace la
 
@@ -59,32 +125,37 @@ extern "C" size_t la_workspace_bytes(int which, int64_t b, int64_t h, int64_t n,
 extern "C" int la_fwd(const void* q, const void* k, const void* v, const float* s, void* o, int64_t b, int64_t h,
                       int64_t n, int64_t d, int64_t e, int dtype, void* workspace, size_t ws_bytes, void* stream) {
     (void)workspace; (void)ws_bytes;
-    int rc = la::check_dims(b, h, n, d, e, dtype);
-    if (rc != LA_OK) return rc;
-    if (b == 0 || n == 0) return LA_OK;  // nothing to do; empty tensors may carry null pointers
-    if (!q || !k || !v || !o) return LA_E_NULLPTR;
-    if (!la::al16(q) || !la::al16(k) || !la::al16(v) || !la::al16(o)) return LA_E_ALIGN;
-    return la::run(q, k, v, o, s, b * h, h, n, d, e, dtype, false, static_cast<hipStream_t>(stream));
+    using la::dense;
+    return la::fwd(dense(q, h, n, d), dense(k, h, n, d), dense(v, h, n, e), s, dense(o, h, n, e), b, h, n, d, e, dtype,
+                   static_cast<hipStream_t>(stream));
 }
 
 extern "C" int la_bwd(const void* q, const void* k, const void* v, const float* s, const void* dout, void* dq,
                       void* dk, void* dv, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
                       void* workspace, size_t ws_bytes, void* stream) {
     (void)workspace; (void)ws_bytes;
-    int rc = la::check_dims(b, h, n, d, e, dtype);
-    if (rc != LA_OK) return rc;
-    if (b == 0 || n == 0) return LA_OK;
-    if (!q || !k || !v || !dout || !dq || !dk || !dv) return LA_E_NULLPTR;
-    if (!la::al16(q) || !la::al16(k) || !la::al16(v) || !la::al16(dout) || !la::al16(dq) || !la::al16(dk) ||
-        !la::al16(dv))
-        return LA_E_ALIGN;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    // dQ_i = sum_{j<=i} lam^(i-j) (dO_i . v_j) k_j
-    rc = la::run(dout, v, k, dq, s, b * h, h, n, e, d, dtype, false, st);
-    if (rc != LA_OK) return rc;
-    // dK_j = sum_{i>=j} lam^(i-j) (v_j . dO_i) q_i
-    rc = la::run(v, dout, q, dk, s, b * h, h, n, e, d, dtype, true, st);
-    if (rc != LA_OK) return rc;
-    // dV_j = sum_{i>=j} lam^(i-j) (k_j . q_i) dO_i
-    return la::run(k, q, dout, dv, s, b * h, h, n, d, e, dtype, true, st);
+    using la::dense;
+    return la::bwd(dense(q, h, n, d), dense(k, h, n, d), dense(v, h, n, e), s, dense(dout, h, n, e), dense(dq, h, n, d),
+                   dense(dk, h, n, d), dense(dv, h, n, e), b, h, n, d, e, dtype, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int la_fwd_strided(const void* q, const void* k, const void* v, const float* s, void* o,
+                              const int64_t* strides, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
+                              void* workspace, size_t ws_bytes, void* stream) {
+    (void)workspace; (void)ws_bytes;
+    if (!strides) return LA_E_NULLPTR;
+    using la::strided;
+    return la::fwd(strided(q, strides), strided(k, strides + 3), strided(v, strides + 6), s, strided(o, strides + 9), b,
+                   h, n, d, e, dtype, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int la_bwd_strided(const void* q, const void* k, const void* v, const float* s, const void* dout, void* dq,
+                              void* dk, void* dv, const int64_t* strides, int64_t b, int64_t h, int64_t n, int64_t d,
+                              int64_t e, int dtype, void* workspace, size_t ws_bytes, void* stream) {
+    (void)workspace; (void)ws_bytes;
+    if (!strides) return LA_E_NULLPTR;
+    using la::strided;
+    return la::bwd(strided(q, strides), strided(k, strides + 3), strided(v, strides + 6), s, strided(dout, strides + 9),
+                   strided(dq, strides + 12), strided(dk, strides + 15), strided(dv, strides + 18), b, h, n, d, e, dtype,
+                   static_cast<hipStream_t>(stream));
 }

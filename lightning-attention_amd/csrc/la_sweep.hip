@@ -76,11 +76,13 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
     const int lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int64_t n = a.n;
     const int dk = a.dk, dv = a.dv;
-    // one bounds-checked buffer per (batch, head) slice: rows >= n read as zero / are not written
-    const __amdgpu_buffer_rsrc_t xb = make_rsrc(static_cast<const T*>(a.x) + (int64_t)unit * n * dk, (unsigned)(n * dk * sizeof(T)));
-    const __amdgpu_buffer_rsrc_t yb = make_rsrc(static_cast<const T*>(a.y) + (int64_t)unit * n * dk, (unsigned)(n * dk * sizeof(T)));
-    const __amdgpu_buffer_rsrc_t zb = make_rsrc(static_cast<const T*>(a.z) + (int64_t)unit * n * dv, (unsigned)(n * dv * sizeof(T)));
-    const __amdgpu_buffer_rsrc_t ob = make_rsrc(static_cast<T*>(a.out) + (int64_t)unit * n * dv, (unsigned)(n * dv * sizeof(T)));
+    // one bounds-checked buffer per (batch, head) sequence; rows >= n are masked by offset below
+    const __amdgpu_buffer_rsrc_t xb = seq_rsrc<T>(a.x, a.lx, unit, a.h, n, dk);
+    const __amdgpu_buffer_rsrc_t yb = seq_rsrc<T>(a.y, a.ly, unit, a.h, n, dk);
+    const __amdgpu_buffer_rsrc_t zb = seq_rsrc<T>(a.z, a.lz, unit, a.h, n, dv);
+    const __amdgpu_buffer_rsrc_t ob = seq_rsrc<T>(a.out, a.lo, unit, a.h, n, dv);
+    const unsigned xts = (unsigned)a.lx.ts, yts = (unsigned)a.ly.ts, zts = (unsigned)a.lz.ts, ots = (unsigned)a.lo.ts;
+    const unsigned nrows = (unsigned)n;
     const int col0 = slice * 64;
     const bool cols_active = (col0 + 16 * w) < dv;
 
@@ -146,27 +148,48 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
     constexpr int NSET = DKP <= 128 ? 2 : 1;
     u32x4 xrA[XC], yrA[XC], zrA, xrB[XC], yrB[XC], zrB;
 
+    // Per-lane byte offsets of this thread's 16-byte chunks inside a 64-token block (out of range
+    // where the chunk lies in the zero padding dk..DKP-1 or beyond dv); the block's first token goes
+    // into the wave-uniform offset of the load.  When a tile row holds a divisor of 512 chunks, a
+    // thread's chunks lie whole rows apart in the same columns and only the first one needs registers.
+    constexpr bool SAMECOL = 512 % (DKP / 8) == 0;
+    constexpr int NLANE = SAMECOL ? 1 : XC;
+    constexpr int CROWS = 512 / (DKP / 8);  // rows between two chunks of a thread (SAMECOL)
+    int lane_row[NLANE];
+    unsigned lane_x[NLANE], lane_y[NLANE];
+#pragma unroll
+    for (int u = 0; u < NLANE; ++u) {
+        const int c = tid + 512 * u;
+        const int row = c / (DKP / 8), col = (c % (DKP / 8)) * 8;
+        lane_row[u] = row;
+        lane_x[u] = col < dk ? (row * xts + col) * (unsigned)sizeof(T) : kOob;
+        lane_y[u] = col < dk ? (row * yts + col) * (unsigned)sizeof(T) : kOob;
+    }
+    const int lane_zrow = tid / 8;
+    const unsigned lane_z = (col0 + (tid % 8) * 8 < dv) ? (lane_zrow * zts + col0 + (tid % 8) * 8) * (unsigned)sizeof(T) : kOob;
     // Fetches block number b of the walk.  Blocks at or beyond it_end, and the x tile of warm-up
     // blocks, are fetched at the out-of-range offset: zeros, no memory traffic, and the sequence of
     // loads is the same on every path.
     auto load_block = [&](int64_t b, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4& zr) {
         const int64_t t = REVERSE ? nblk - 1 - b : b;
         const bool valid = b < it_end, need_x = valid && b >= it_first;
-        const unsigned tok0 = (unsigned)(t * 64);
+        const unsigned tok0 = valid ? (unsigned)(t * 64) : 0u;
+        // rows of this block that exist (0 for a block that is not fetched)
+        const int rows = valid ? (int)min(64u, nrows - tok0) : 0, rows_x = need_x ? rows : 0;
 #pragma unroll
         for (int u = 0; u < XC; ++u) {
-            const int c = tid + 512 * u;
-            const int row = c / (DKP / 8), col = (c % (DKP / 8)) * 8;
-            // columns dk..DKP-1 are zero padding
-            const unsigned off = col < dk ? ((tok0 + row) * (unsigned)dk + col) * (unsigned)sizeof(T) : kOob;
-            xr[u] = buf_load16(xb, need_x ? off : kOob);
-            yr[u] = buf_load16(yb, valid ? off : kOob);
+            if (SAMECOL) {
+                // a wave-uniform offset must stay inside the buffer: 0 when none of these rows exists
+                const unsigned tk = u * CROWS < rows ? tok0 + u * CROWS : 0u;
+                xr[u] = buf_load16(xb, lane_row[0] < rows_x - u * CROWS ? lane_x[0] : kOob, tk * xts * (unsigned)sizeof(T));
+                yr[u] = buf_load16(yb, lane_row[0] < rows - u * CROWS ? lane_y[0] : kOob, tk * yts * (unsigned)sizeof(T));
+            } else {
+                const int v = u < NLANE ? u : 0;
+                xr[u] = buf_load16(xb, lane_row[v] < rows_x ? lane_x[v] : kOob, tok0 * xts * (unsigned)sizeof(T));
+                yr[u] = buf_load16(yb, lane_row[v] < rows ? lane_y[v] : kOob, tok0 * yts * (unsigned)sizeof(T));
+            }
         }
-        {
-            const int row = tid / 8, col = (tid % 8) * 8;
-            const unsigned off = (col0 + col < dv) ? ((tok0 + row) * (unsigned)dv + col0 + col) * (unsigned)sizeof(T) : kOob;
-            zr = buf_load16(zb, valid ? off : kOob);
-        }
+        zr = buf_load16(zb, lane_zrow < rows ? lane_z : kOob, tok0 * zts * (unsigned)sizeof(T));
     };
     auto stage_block = [&](int buf, const u32x4 (&xr)[XC], const u32x4 (&yr)[XC], const u32x4& zr) {
         T* Xd = tiles + buf * L::TILE;
@@ -362,12 +385,12 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
                 const int col = col0 + 16 * w + 4 * g;
 #pragma unroll
                 for (int i4 = 0; i4 < 4; ++i4) {
-                    const unsigned tok = (unsigned)(t * 64) + 16 * i4 + r;
+                    const unsigned tok = (unsigned)(t * 64) + 16 * i4;  // wave-uniform first token of the tile
                     V4 o;
 #pragma unroll
                     for (int v = 0; v < 4; ++v) o[v] = (T)oacc[i4][v];
-                    const unsigned off = col < dv ? (tok * (unsigned)dv + col) * (unsigned)sizeof(T) : kOob;
-                    buf_store8(ob, off, __builtin_bit_cast(u32x2, o));
+                    const unsigned off = (col < dv && tok + r < nrows) ? (r * ots + col) * (unsigned)sizeof(T) : kOob;
+                    buf_store8(ob, off, tok < nrows ? tok * ots * (unsigned)sizeof(T) : 0u, __builtin_bit_cast(u32x2, o));
                 }
             }
         } else if (cols_active && have_next) {
@@ -505,11 +528,13 @@ static void choose_chunks(SweepArgs& a) {
     for (int i = (int)c + 1; i < 9; ++i) a.chunk_start[i] = (int)nblk;
 }
 
-// x,y: (bh,n,dk)  z,out: (bh,n,dv)
-int sweep(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h, int64_t n,
-          int64_t dk, int64_t dv, int dtype, bool reverse, hipStream_t st) {
+// x,y: (b,h,n,dk)  z,out: (b,h,n,dv), each with its own batch / head / token strides
+int sweep(const void* x, const void* y, const void* z, void* out, const Layout& lx, const Layout& ly, const Layout& lz,
+          const Layout& lo, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
+          bool reverse, hipStream_t st) {
     SweepArgs a;
     a.x = x; a.y = y; a.z = z; a.out = out; a.s = s;
+    a.lx = lx; a.ly = ly; a.lz = lz; a.lo = lo;
     a.n = n; a.dk = (int)dk; a.dv = (int)dv; a.h = (int)h; a.bh = (int)bh;
     a.nslice = (int)((dv + 63) / 64);
     choose_chunks(a);

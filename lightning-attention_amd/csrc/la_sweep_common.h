@@ -4,17 +4,32 @@
 
 namespace la {
 
+// Where the (batch, head, token) rows of a tensor start, in elements; the feature dim is contiguous.
+// A plain (b, h, n, d) tensor has {h*n*d, n*d, d}; a (b, n, h, d) projection output viewed as
+// (b, h, n, d) has {n*h*d, d, h*d}.
+struct Layout {
+    int64_t bs, hs, ts;  // batch, head, token stride
+};
+
 struct SweepArgs {
-    const void* x;  // (bh, n, dk)
-    const void* y;  // (bh, n, dk)
-    const void* z;  // (bh, n, dv)
-    void* out;      // (bh, n, dv)
+    const void* x;  // (b, h, n, dk)
+    const void* y;  // (b, h, n, dk)
+    const void* z;  // (b, h, n, dv)
+    void* out;      // (b, h, n, dv)
+    Layout lx, ly, lz, lo;
     const float* s; // h decay rates or nullptr
     int64_t n;
     int dk, dv, h, bh, nslice;
     int nchunk;          // sequence chunks per (batch, head, slice); 1 = one workgroup walks the whole sequence
     int chunk_start[9];  // first 64-token block (in walk order) of each chunk; chunk_start[nchunk] = number of blocks
 };
+
+// Bounds-checked buffer over the rows of one (batch, head) sequence of a tensor with `cols` features.
+template <typename T>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t seq_rsrc(const void* p, const Layout& l, int unit, int h, int64_t n, int cols) {
+    const T* base = static_cast<const T*>(p) + (int64_t)(unit / h) * l.bs + (int64_t)(unit % h) * l.hs;
+    return make_rsrc(base, (unsigned)(((n - 1) * l.ts + cols) * (int64_t)sizeof(T)));
+}
 
 template <typename T>
 struct Mma;

@@ -82,11 +82,13 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepArgs a) {
     const int lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int64_t n = a.n;
     const int dk = a.dk, dv = a.dv;
-    // one bounds-checked buffer per (batch, head) slice: rows >= n read as zero / are not written
-    const __amdgpu_buffer_rsrc_t xb = make_rsrc(static_cast<const T*>(a.x) + (int64_t)unit * n * dk, (unsigned)(n * dk * sizeof(T)));
-    const __amdgpu_buffer_rsrc_t yb = make_rsrc(static_cast<const T*>(a.y) + (int64_t)unit * n * dk, (unsigned)(n * dk * sizeof(T)));
-    const __amdgpu_buffer_rsrc_t zb = make_rsrc(static_cast<const T*>(a.z) + (int64_t)unit * n * dv, (unsigned)(n * dv * sizeof(T)));
-    const __amdgpu_buffer_rsrc_t ob = make_rsrc(static_cast<T*>(a.out) + (int64_t)unit * n * dv, (unsigned)(n * dv * sizeof(T)));
+    // one bounds-checked buffer per (batch, head) sequence; rows >= n are masked by offset below
+    const __amdgpu_buffer_rsrc_t xb = seq_rsrc<T>(a.x, a.lx, unit, a.h, n, dk);
+    const __amdgpu_buffer_rsrc_t yb = seq_rsrc<T>(a.y, a.ly, unit, a.h, n, dk);
+    const __amdgpu_buffer_rsrc_t zb = seq_rsrc<T>(a.z, a.lz, unit, a.h, n, dv);
+    const __amdgpu_buffer_rsrc_t ob = seq_rsrc<T>(a.out, a.lo, unit, a.h, n, dv);
+    const unsigned xts = (unsigned)a.lx.ts, yts = (unsigned)a.ly.ts, zts = (unsigned)a.lz.ts, ots = (unsigned)a.lo.ts;
+    const unsigned nrows = (unsigned)n;
     const int col0 = slice * 64;
     const bool cols_active = (col0 + 16 * w) < dv;
 
@@ -149,6 +151,16 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepArgs a) {
 
     u32x4 xrA[XC], yrA[XC], zrA, xrB[XC], yrB[XC], zrB;
 
+    // Per-lane byte offsets of this thread's first 16-byte chunk inside a 64-token block (out of
+    // range where the chunk lies in the zero padding dk..DKP-1 or beyond dv).  Its further chunks
+    // lie a whole number of rows below, so they and the block's first token go into the
+    // wave-uniform offset of the load.
+    constexpr int CROWS = 512 / (DKP / 8);  // rows between two chunks of a thread
+    const int lane_row = tid / (DKP / 8), lane_col = (tid % (DKP / 8)) * 8;
+    const unsigned lane_x = lane_col < dk ? (lane_row * xts + lane_col) * (unsigned)sizeof(T) : kOob;
+    const unsigned lane_y = lane_col < dk ? (lane_row * yts + lane_col) * (unsigned)sizeof(T) : kOob;
+    const int lane_zrow = tid / 8;
+    const unsigned lane_z = (col0 + (tid % 8) * 8 < dv) ? (lane_zrow * zts + col0 + (tid % 8) * 8) * (unsigned)sizeof(T) : kOob;
     // Fetches block number b of the walk.  Blocks at or beyond it_end, and the x tile of warm-up
     // blocks, are fetched at the out-of-range offset: zeros, no memory traffic, and the sequence of
     // memory operations is the same for every wave on every path (the waits the compiler places
@@ -156,21 +168,17 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepArgs a) {
     auto load_block = [&](int64_t b, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4& zr) {
         const int64_t t = REVERSE ? nblk - 1 - b : b;
         const bool valid = b < it_end, need_x = valid && b >= it_first;
-        const unsigned tok0 = (unsigned)(t * 64);
+        const unsigned tok0 = valid ? (unsigned)(t * 64) : 0u;
+        // rows of this block that exist (0 for a block that is not fetched)
+        const int rows = valid ? (int)min(64u, nrows - tok0) : 0, rows_x = need_x ? rows : 0;
 #pragma unroll
         for (int u = 0; u < XC; ++u) {
-            const int c = tid + 512 * u;
-            const int row = c / (DKP / 8), col = (c % (DKP / 8)) * 8;
-            // columns dk..DKP-1 are zero padding
-            const unsigned off = col < dk ? ((tok0 + row) * (unsigned)dk + col) * (unsigned)sizeof(T) : kOob;
-            xr[u] = buf_load16(xb, need_x ? off : kOob);
-            yr[u] = buf_load16(yb, valid ? off : kOob);
+            // a wave-uniform offset must stay inside the buffer: 0 when none of these rows exists
+            const unsigned tk = u * CROWS < rows ? tok0 + u * CROWS : 0u;
+            xr[u] = buf_load16(xb, lane_row < rows_x - u * CROWS ? lane_x : kOob, tk * xts * (unsigned)sizeof(T));
+            yr[u] = buf_load16(yb, lane_row < rows - u * CROWS ? lane_y : kOob, tk * yts * (unsigned)sizeof(T));
         }
-        {
-            const int row = tid / 8, col = (tid % 8) * 8;
-            const unsigned off = (col0 + col < dv) ? ((tok0 + row) * (unsigned)dv + col0 + col) * (unsigned)sizeof(T) : kOob;
-            zr = buf_load16(zb, valid ? off : kOob);
-        }
+        zr = buf_load16(zb, lane_zrow < rows ? lane_z : kOob, tok0 * zts * (unsigned)sizeof(T));
     };
     const unsigned lane_stage_xy = ((tid / (DKP / 8)) * XS + (tid % (DKP / 8)) * 8) * E;
     const unsigned lane_stage_z = ((tid / 8) * ZS + (tid % 8) * 8) * E;
@@ -366,12 +374,12 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepArgs a) {
                 const int col = col0 + 16 * w + 4 * g;
 #pragma unroll
                 for (int i4 = 0; i4 < 4; ++i4) {
-                    const unsigned tok = (unsigned)(t * 64) + 16 * i4 + r;
+                    const unsigned tok = (unsigned)(t * 64) + 16 * i4;  // wave-uniform first token of the tile
                     V4 o;
 #pragma unroll
                     for (int v = 0; v < 4; ++v) o[v] = (T)oacc[i4][v];
-                    const unsigned off = col < dv ? (tok * (unsigned)dv + col) * (unsigned)sizeof(T) : kOob;
-                    buf_store8(ob, off, __builtin_bit_cast(u32x2, o));
+                    const unsigned off = (col < dv && tok + r < nrows) ? (r * ots + col) * (unsigned)sizeof(T) : kOob;
+                    buf_store8(ob, off, tok < nrows ? tok * ots * (unsigned)sizeof(T) : 0u, __builtin_bit_cast(u32x2, o));
                 }
             } else {
                 dummy_stores();

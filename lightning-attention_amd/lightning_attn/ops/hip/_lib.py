@@ -16,7 +16,7 @@ _DTYPES = {torch.bfloat16: LA_BF16, torch.float16: LA_FP16, torch.float32: LA_FP
 
 SYMBOLS = (
     "la_version", "la_error_string", "la_supported", "la_workspace_bytes",
-    "la_fwd", "la_bwd", "srmsnorm_fwd", "srmsnorm_bwd",
+    "la_fwd", "la_bwd", "la_fwd_strided", "la_bwd_strided", "srmsnorm_fwd", "srmsnorm_bwd",
 )
 
 _lib = None
@@ -50,6 +50,11 @@ def lib():
             L.la_bwd.restype = _int
             L.la_bwd.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
                                  _vp, _sz, _vp]
+            L.la_fwd_strided.restype = _int
+            L.la_fwd_strided.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]
+            L.la_bwd_strided.restype = _int
+            L.la_bwd_strided.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
+                                         _int, _vp, _sz, _vp]
             L.srmsnorm_fwd.restype = _int
             L.srmsnorm_fwd.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _f, _int, _vp]
             L.srmsnorm_bwd.restype = _int

@@ -3,54 +3,101 @@
 Same names and call conventions as lightning_attn/ops/triton/lightning_attn2.py:398-507
 and lightning_attn2_no_decay.py:367-471: ``lightning_attn2(q, k, v, s)`` and
 ``lightning_attn2_no_decay(q, k, v)`` with q,k (b,h,n,d), v (b,h,n,e), s holding
-h float32 rates; inputs are made contiguous, outputs come from torch.empty,
-kernels go on the current stream, and only the inputs are saved for backward."""
+h float32 rates; outputs come from torch.empty, kernels go on the current stream,
+and only the inputs are saved for backward.
+
+Where the reference copies (``.contiguous()`` on q, k, v, do, lightning_attn2.py:402-405,
+439-442), bf16 / fp16 tensors whose feature dim is contiguous and whose other strides are
+16-byte multiples are used in place: a projection output ``(b, n, h*d)`` viewed as
+``(b, h, n, d)`` needs no copy, and o, dq, dk, dv are allocated in the memory order of
+v, q, k, v, so ``rearrange(o, "b h n d -> b n (h d)")`` is a view as well."""
+import ctypes
+
 import torch
 
 from . import _lib
 
 
+def _in_place_ok(t):
+    """True when the kernels can address `t` (b,h,n,c) through its own strides."""
+    if t.dtype == torch.float32 or t.dim() != 4 or t.stride(3) != 1:
+        return False
+    elt = t.element_size()
+    if t.data_ptr() % 16:
+        return False
+    for i in range(3):
+        if t.stride(i) < 0 or (t.stride(i) * elt) % 16:
+            return False
+        if t.shape[i] > 1 and t.stride(i) == 0:
+            return False
+    if t.stride(2) < t.shape[3]:
+        return False
+    return ((t.shape[2] - 1) * t.stride(2) + t.shape[3]) * elt < 2 ** 31
+
+
+def _usable(t):
+    return t if (t.is_contiguous() or _in_place_ok(t)) else t.contiguous()
+
+
+def _strides(*tensors):
+    vals = []
+    for t in tensors:
+        vals += [t.stride(0), t.stride(1), t.stride(2)]
+    return (ctypes.c_int64 * len(vals))(*vals)
+
+
 def _fwd(q, k, v, s):
     _lib.require_gpu(q, "lightning_attn2")
-    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     if not (q.dtype == k.dtype == v.dtype):
         raise TypeError("q, k, v must share a dtype")
+    if q.dim() != 4 or k.shape != q.shape or v.dim() != 4 or v.shape[:3] != q.shape[:3]:
+        raise ValueError("shape mismatch: q %s k %s v %s" % (tuple(q.shape), tuple(k.shape), tuple(v.shape)))
+    q, k, v = _usable(q), _usable(k), _usable(v)
     b, h, n, d = q.shape
     e = v.shape[-1]
-    if k.shape != q.shape or v.shape[:3] != q.shape[:3]:
-        raise ValueError("shape mismatch: q %s k %s v %s" % (tuple(q.shape), tuple(k.shape), tuple(v.shape)))
     if s is not None:
         s = s.to(device=q.device, dtype=torch.float32).contiguous()
         if s.numel() != h:
             raise ValueError("s must hold one rate per head (%d), got %d" % (h, s.numel()))
     L = _lib.lib()
     code = _lib.dtype_code(q.dtype)
-    o = torch.empty((b, h, n, e), dtype=q.dtype, device=q.device)
+    o = torch.empty_like(v)  # same sizes as v; dense, in v's memory order
     ws_bytes = L.la_workspace_bytes(0, b, h, n, d, e, code)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
+    sp = s.data_ptr() if s is not None else None
+    wp = ws.data_ptr() if ws is not None else None
     with torch.cuda.device(q.device):
-        rc = L.la_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr() if s is not None else None,
-                      o.data_ptr(), b, h, n, d, e, code, ws.data_ptr() if ws is not None else None, ws_bytes,
-                      _lib.stream_ptr(q.device))
+        if all(t.is_contiguous() for t in (q, k, v, o)):
+            rc = L.la_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, o.data_ptr(), b, h, n, d, e, code, wp, ws_bytes,
+                          _lib.stream_ptr(q.device))
+        else:
+            rc = L.la_fwd_strided(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, o.data_ptr(), _strides(q, k, v, o),
+                                  b, h, n, d, e, code, wp, ws_bytes, _lib.stream_ptr(q.device))
     _lib.check(rc, "la_fwd")
     return o, q, k, v, s
 
 
 def _bwd(q, k, v, s, do):
-    do = do.contiguous()
     b, h, n, d = q.shape
     e = v.shape[-1]
     L = _lib.lib()
     code = _lib.dtype_code(q.dtype)
     if do.dtype != q.dtype:
         do = do.to(q.dtype)
+    do = _usable(do)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     ws_bytes = L.la_workspace_bytes(1, b, h, n, d, e, code)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
+    sp = s.data_ptr() if s is not None else None
+    wp = ws.data_ptr() if ws is not None else None
     with torch.cuda.device(q.device):
-        rc = L.la_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr() if s is not None else None,
-                      do.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), b, h, n, d, e, code,
-                      ws.data_ptr() if ws is not None else None, ws_bytes, _lib.stream_ptr(q.device))
+        if all(t.is_contiguous() for t in (q, k, v, do, dq, dk, dv)):
+            rc = L.la_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, do.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                          dv.data_ptr(), b, h, n, d, e, code, wp, ws_bytes, _lib.stream_ptr(q.device))
+        else:
+            rc = L.la_bwd_strided(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, do.data_ptr(), dq.data_ptr(),
+                                  dk.data_ptr(), dv.data_ptr(), _strides(q, k, v, do, dq, dk, dv), b, h, n, d, e, code,
+                                  wp, ws_bytes, _lib.stream_ptr(q.device))
     _lib.check(rc, "la_bwd")
     return dq, dk, dv
 

@@ -160,6 +160,41 @@ def test_strided_inputs_and_slope_layouts():
         assert torch.equal(a, c)
 
 
+@pytest.mark.parametrize("b, h, n, d, e", [(2, 4, 300, 128, 128), (1, 3, 1111, 64, 96), (2, 12, 257, 192, 192)])
+def test_projection_layout_is_used_in_place(b, h, n, d, e):
+    """q, k, v sliced out of one fused (b, n, 3*h*d)-style projection and viewed as (b, h, n, d): the strided entry
+    points read them where they are, write o / dq / dk / dv in token-major order (so that
+    "b h n d -> b n (h d)" is a view), and give bit-identical values to the plain-layout call."""
+    g = torch.Generator().manual_seed(11)
+    fused = torch.randn(b, n, h * (2 * d + e), generator=g).bfloat16().to(DEV)
+    do_nm = torch.randn(b, n, h * e, generator=g).bfloat16().to(DEV)
+    s = _build_slope_tensor(h).to(DEV)
+    qs, ks, vs = fused.split([h * d, h * d, h * e], dim=-1)
+    views = [t.unflatten(-1, (h, -1)).transpose(1, 2) for t in (qs, ks, vs)]
+    assert not any(t.is_contiguous() for t in views)
+    qv, kv, vv = (t.detach().requires_grad_() for t in views)
+    produced = []  # gradients as the operator's backward hands them over (before autograd accumulates them)
+    for t in (qv, kv, vv):
+        t.register_hook(produced.append)
+    o = lightning_attn_func(qv, kv, vv, s)
+    assert o.shape == (b, h, n, e) and o.transpose(1, 2).is_contiguous()
+    o.backward(do_nm.unflatten(-1, (h, e)).transpose(1, 2))
+    assert len(produced) == 3
+    for t in produced:
+        assert t.transpose(1, 2).is_contiguous()
+    # the same numbers through the plain (b, h, n, d) layout
+    qc, kc, vc = (t.detach().contiguous().requires_grad_() for t in views)
+    oc = lightning_attn_func(qc, kc, vc, s)
+    assert oc.is_contiguous()
+    oc.backward(do_nm.unflatten(-1, (h, e)).transpose(1, 2).contiguous())
+    torch.cuda.synchronize()
+    for a, c in zip((o, qv.grad, kv.grad, vv.grad), (oc, qc.grad, kc.grad, vc.grad)):
+        assert torch.equal(a, c)
+    want = oracle.linear_attn_fwd_bwd(qc.detach().cpu(), kc.detach().cpu(), vc.detach().cpu(), s.cpu(),
+                                      do_nm.unflatten(-1, (h, e)).transpose(1, 2).cpu(), torch.float32)
+    check((o.detach(), qv.grad, kv.grad, vv.grad), want, torch.bfloat16, "projection layout")
+
+
 def test_wide_features_are_split_by_the_interface():
     """d, e above the kernels' 256 limit go through the slice-and-add path of lightning_attn_func."""
     q, k, v, do = make_inputs(1, 2, 200, 320, 264, torch.bfloat16, 0.5)

@@ -51,6 +51,22 @@ def test_host_only_entry_points():
     assert L.srmsnorm_fwd(p16, p16, p16, 4, 0, 64, 1e-6, 0, None) == -2
     assert L.srmsnorm_fwd(p16, p16, p16, 4, 64, 32, 1e-6, 0, None) == -2
     assert L.srmsnorm_fwd(p16, p16, p16, 4, 64, 64, 1e-6, 9, None) == -3
+    # strided entry points: strides in elements, (batch, head, token) per tensor
+    dense = [64 * 64, 64 * 64, 64] * 4
+    def st(vals):
+        return (ctypes.c_int64 * len(vals))(*vals)
+    assert L.la_fwd_strided(p16, p16, p16, None, p16, None, 1, 1, 64, 64, 64, 0, None, 0, None) == -1
+    assert L.la_fwd_strided(None, p16, p16, None, p16, st(dense), 1, 1, 64, 64, 64, 0, None, 0, None) == -1
+    bad = list(dense); bad[2] = 68  # token stride not a multiple of 16 bytes
+    assert L.la_fwd_strided(p16, p16, p16, None, p16, st(bad), 1, 1, 64, 64, 64, 0, None, 0, None) == -5
+    bad = list(dense); bad[5] = 32  # token stride below the feature dim
+    assert L.la_fwd_strided(p16, p16, p16, None, p16, st(bad), 1, 1, 64, 64, 64, 0, None, 0, None) == -2
+    bad = list(dense); bad[11] = 1 << 26  # one sequence would span more than 2 GiB
+    assert L.la_fwd_strided(p16, p16, p16, None, p16, st(bad), 1, 1, 64, 64, 64, 0, None, 0, None) == -2
+    bad = list(dense); bad[2] = 128  # float32 tensors must be plain
+    assert L.la_fwd_strided(p16, p16, p16, None, p16, st(bad), 1, 1, 64, 64, 64, 2, None, 0, None) == -3
+    assert L.la_bwd_strided(p16, p16, p16, None, p16, p16, p16, p16, None, 1, 1, 64, 64, 64, 0, None, 0, None) == -1
+    assert L.la_fwd_strided(p16, p16, p16, None, p16, st(dense), 0, 4, 64, 64, 64, 0, None, 0, None) == 0
     # empty problems succeed without touching the device
     assert L.la_fwd(p16, p16, p16, None, p16, 0, 4, 64, 64, 64, 0, None, 0, None) == 0
     assert L.srmsnorm_bwd(p16, p16, p16, p16, 0, 64, 64, 0, None) == 0
