@@ -18,6 +18,16 @@ import torch
 from . import _lib
 
 
+def _norm_strides(t):
+    """Strides of a 4-d tensor with those of size-1 dims (never used for addressing, may be
+    anything) replaced by the dense value."""
+    st = list(t.stride())
+    for i in (2, 1, 0):
+        if t.shape[i] == 1:
+            st[i] = t.shape[i + 1] * st[i + 1]
+    return st
+
+
 def _in_place_ok(t):
     """True when the kernels can address `t` (b,h,n,c) through its own strides."""
     if t.dtype == torch.float32 or t.dim() != 4 or t.stride(3) != 1:
@@ -25,14 +35,12 @@ def _in_place_ok(t):
     elt = t.element_size()
     if t.data_ptr() % 16:
         return False
-    for i in range(3):
-        if t.stride(i) < 0 or (t.stride(i) * elt) % 16:
-            return False
-        if t.shape[i] > 1 and t.stride(i) == 0:
-            return False
-    if t.stride(2) < t.shape[3]:
+    st = _norm_strides(t)
+    if any(x <= 0 or (x * elt) % 16 for x in st[:3]):
         return False
-    return ((t.shape[2] - 1) * t.stride(2) + t.shape[3]) * elt < 2 ** 31
+    if st[2] < t.shape[3]:
+        return False
+    return ((t.shape[2] - 1) * st[2] + t.shape[3]) * elt < 2 ** 31
 
 
 def _usable(t):
@@ -40,9 +48,10 @@ def _usable(t):
 
 
 def _strides(*tensors):
+    """(batch, head, token) strides of each tensor, in argument order."""
     vals = []
     for t in tensors:
-        vals += [t.stride(0), t.stride(1), t.stride(2)]
+        vals += _norm_strides(t)[:3]
     return (ctypes.c_int64 * len(vals))(*vals)
 
 

@@ -195,6 +195,25 @@ def test_projection_layout_is_used_in_place(b, h, n, d, e):
     check((o.detach(), qv.grad, kv.grad, vv.grad), want, torch.bfloat16, "projection layout")
 
 
+def test_mixed_layouts_and_unit_dims():
+    """One plain tensor whose size-1 batch dim carries an odd stride, one token-major view, one head-sliced
+    view of a wider tensor: every tensor keeps its own layout in the same call."""
+    h, n, d, e = 4, 200, 64, 64
+    g = torch.Generator().manual_seed(17)
+    q = (torch.randn(1, h, n, d, generator=g) * 0.5).bfloat16().to(DEV)
+    q = q.as_strided(q.shape, (7, n * d, d, 1))                      # the batch stride is never used
+    k = (torch.randn(1, n, h, d, generator=g) * 0.5).bfloat16().to(DEV).transpose(1, 2)
+    v = (torch.randn(1, h + 2, n, e, generator=g) * 0.5).bfloat16().to(DEV)[:, 1:h + 1]
+    do = torch.randn(1, n, h, e, generator=g).bfloat16().to(DEV).transpose(1, 2)
+    s = _build_slope_tensor(h).to(DEV)
+    qg, kg, vg = (t.detach().requires_grad_() for t in (q, k, v))
+    o = lightning_attn_func(qg, kg, vg, s)
+    o.backward(do)
+    torch.cuda.synchronize()
+    want = oracle.linear_attn_fwd_bwd(q.cpu(), k.cpu(), v.cpu(), s.cpu(), do.cpu(), torch.float32)
+    check((o.detach(), qg.grad, kg.grad, vg.grad), want, torch.bfloat16, "mixed layouts")
+
+
 def test_wide_features_are_split_by_the_interface():
     """d, e above the kernels' 256 limit go through the slice-and-add path of lightning_attn_func."""
     q, k, v, do = make_inputs(1, 2, 200, 320, 264, torch.bfloat16, 0.5)
