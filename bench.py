@@ -43,6 +43,11 @@ def bytes_per_token(d, e, which, elt=2):
     return {"fwd": fwd, "bwd": bwd, "both": fwd + bwd}[which]
 
 
+def _clear(*tensors):
+    for t in tensors:
+        t.grad = None
+
+
 def event_ms(fn, reps, warm=3):
     """Average duration of fn() over reps launches, HIP events on the current stream
     (the stream the operators launch on)."""
@@ -213,6 +218,25 @@ def main():
             q, k, v, do = inputs(n)
             sweep[str(n)] = round(event_ms(step, 10 if n >= 16384 else 20), 4)
         out["n_sweep_fwd_bwd_ms"] = sweep
+        # the other GPU configurations (parity-test cases; timings for reference only):
+        # configs[1] without decay, config 4 = b2 h12 n2048 d=e=192 with and without decay, and config 4's
+        # shape fed token-major (a (b, n, h*d) projection output used in place through the strided entry points)
+        q = k = v = do = None
+        extra = {}
+        q, k, v, do = inputs(4096)
+        extra["b4_h32_n4096_d128_no_decay_ms"] = round(event_ms(lambda: (lightning_attn_func(q, k, v, None).backward(do), _clear(q, k, v)), 20), 4)
+        q = k = v = do = None
+        b4, h4, n4, d4 = 2, 12, 2048, 192
+        s4 = _build_slope_tensor(h4).to(dev).to(torch.float32)
+        q, k, v, do = (torch.randn(b4, h4, n4, d4, device=dev).bfloat16() for _ in range(4))
+        q, k, v = q.requires_grad_(), k.requires_grad_(), v.requires_grad_()
+        extra["b2_h12_n2048_d192_ms"] = round(event_ms(lambda: (lightning_attn_func(q, k, v, s4).backward(do), _clear(q, k, v)), 30), 4)
+        extra["b2_h12_n2048_d192_no_decay_ms"] = round(event_ms(lambda: (lightning_attn_func(q, k, v, None).backward(do), _clear(q, k, v)), 30), 4)
+        qt, kt, vt = (torch.randn(b4, n4, h4, d4, device=dev).bfloat16().transpose(1, 2).requires_grad_() for _ in range(3))
+        dot = torch.randn(b4, n4, h4, d4, device=dev).bfloat16().transpose(1, 2)
+        extra["b2_h12_n2048_d192_token_major_ms"] = round(event_ms(lambda: (lightning_attn_func(qt, kt, vt, s4).backward(dot), _clear(qt, kt, vt)), 30), 4)
+        out["other_configs_fwd_bwd"] = extra
+        qt = kt = vt = dot = None
     del q, k, v, do
     if not args.no_srms:
         # SRMSNorm, config 5: [32768, 4096] bf16, 1 % outliers x50
