@@ -32,6 +32,9 @@ __device__ __forceinline__ u32x4 buf_load16(__amdgpu_buffer_rsrc_t r, unsigned o
 __device__ __forceinline__ void buf_store8(__amdgpu_buffer_rsrc_t r, unsigned off, u32x2 v) {
     __builtin_amdgcn_raw_buffer_store_b64(v, r, off, 0, 0);
 }
+__device__ __forceinline__ void buf_store16(__amdgpu_buffer_rsrc_t r, unsigned off, unsigned soff, u32x4 v) {
+    __builtin_amdgcn_raw_buffer_store_b128(v, r, off, soff, 0);
+}
 // The same with a wave-uniform byte offset `soff` added to the per-lane one.  `soff` must lie
 // inside the buffer (the hardware compares the per-lane offset with the range left after it).
 __device__ __forceinline__ u32x4 buf_load16(__amdgpu_buffer_rsrc_t r, unsigned off, unsigned soff) {

@@ -5,18 +5,24 @@
 // 8 wavefronts per (batch, head, 64-column slice of z/out), 64-token blocks walked in
 // order, fp32 state in MFMA accumulators), but the two kinds of wavefronts work on
 // different blocks at the same time:
-//   waves 0-3 ("score" waves)  during iteration `it` they compute the masked, decayed
-//                              score tile P of block it+1 and leave it in LDS;
+//   waves 0-3 ("score" waves)  do all the memory traffic (fetch blocks it+3 / it+4 into two
+//                              register sets, publish block it+2 in LDS, write the output
+//                              tile of block it-1 back) and, during iteration `it`, compute
+//                              the masked, decayed score tile P of block it+1 into LDS;
 //   waves 4-7 ("state" waves)  own a dk x 16 column slab of the state and finish block
-//                              `it`: out^T = Lout * (state^T x^T) + z^T P^T, store, then
-//                              state = lam^64 state + y^T (z * Lupd).
-// The inter-block term therefore never leaves registers, nothing is handed from one kind of
-// wave to the other inside an iteration, and a single barrier per iteration orders
+//                              `it`: out^T = Lout * (state^T x^T) + z^T P^T, left in LDS,
+//                              then state = lam^64 state + y^T (z * Lupd).
+// The inter-block term therefore never leaves registers, the state waves' serial chain holds
+// no memory instructions, and a single barrier per iteration orders
 //   - the x/y/z tiles: three LDS buffers (block `it` read by the state waves, block it+1
-//     read by the score waves, block it+2 being written), fed from two register sets so that
-//     blocks it+3 and it+4 are in flight from memory;
-//   - the P tiles: two LDS buffers (block `it` read, block it+1 written).
+//     read by the score waves, block it+2 being written);
+//   - the P tiles: two LDS buffers (block `it` read, block it+1 written);
+//   - the output tile of block `it`, which the state waves write over the z columns they
+//     alone read and which leaves for memory as whole 128-byte row segments when that z slot
+//     is refilled one iteration later.
 // (lightning_attn/ops/triton/lightning_attn2.py:8-85 forward, :88-395 backward.)
+#include <type_traits>
+
 #include "la_sweep_common.h"
 #include "lightning_attn_hip.h"
 
@@ -50,7 +56,14 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepArgs a) {
     constexpr int XS = L::XS, ZS = L::ZS, PS = L::PS;
     constexpr int KS = DKP / 32;  // 32-wide contraction steps over the feature dim
     constexpr int KT = DKP / 16;  // 16-row state tiles
-    constexpr int XC = DKP / 64;  // 16-byte chunks per thread for an x / y tile (512 threads)
+#ifndef LA_PIPE_LOADERS
+#define LA_PIPE_LOADERS 256
+#endif
+    // Threads that fetch, publish and write back the tiles: the 256 of the score waves, which have
+    // slack; the state waves' serial chain then holds no memory instructions at all.
+    constexpr int NL = LA_PIPE_LOADERS;
+    constexpr int XC = 64 * (DKP / 8) / NL;  // 16-byte chunks per loader thread for an x / y tile
+    constexpr int ZC = 512 / NL;             // ... and for the z slice / the output tile
     extern __shared__ __align__(16) unsigned char smem[];
     // LDS map in bytes: [3][x 64*XS | y 64*XS] tiles, [3][64*ZS] z tiles, [2][64*PS] P tiles.
     // All LDS accesses below are written as (per-iteration base register) + (compile-time
@@ -151,13 +164,14 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepArgs a) {
     const int64_t it_first = a.chunk_start[chunk];
     const int64_t it_end = a.chunk_start[chunk + 1];
 
-    u32x4 xrA[XC], yrA[XC], zrA, xrB[XC], yrB[XC], zrB;
+    u32x4 xrA[XC], yrA[XC], zrA[ZC], xrB[XC], yrB[XC], zrB[ZC];
+    const bool loader = tid < NL;
 
     // Per-lane byte offsets of this thread's first 16-byte chunk inside a 64-token block (out of
     // range where the chunk lies in the zero padding dk..DKP-1 or beyond dv).  Its further chunks
     // lie a whole number of rows below, so they and the block's first token go into the
     // wave-uniform offset of the load.
-    constexpr int CROWS = 512 / (DKP / 8);  // rows between two chunks of a thread
+    constexpr int CROWS = NL / (DKP / 8);  // rows between two chunks of a thread
     const int lane_row = tid / (DKP / 8), lane_col = (tid % (DKP / 8)) * 8;
     const unsigned lane_x = lane_col < dk ? (lane_row * xts + lane_col) * (unsigned)sizeof(T) : kOob;
     const unsigned lane_y = lane_col < dk ? (lane_row * yts + lane_col) * (unsigned)sizeof(T) : kOob;
@@ -166,7 +180,7 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepArgs a) {
     // Fetches block number b of the walk.  Blocks at or beyond it_end, and the x tile of warm-up
     // blocks, are fetched at the out-of-range offset: zeros, no memory traffic, and the loads are
     // issued unconditionally (no branches, no draining `s_waitcnt vmcnt(0)` at joins).
-    auto load_block = [&](int64_t b, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4& zr) {
+    auto load_block = [&](int64_t b, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4 (&zr)[ZC]) {
         const int64_t t = REVERSE ? nblk - 1 - b : b;
         const bool valid = b < it_end, need_x = valid && b >= it_first;
         if (DENSE) {
@@ -177,15 +191,18 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepArgs a) {
             const unsigned tok0 = (unsigned)(t * 64);
 #pragma unroll
             for (int u = 0; u < XC; ++u) {
-                const int c = tid + 512 * u;
+                const int c = tid + NL * u;
                 const int row = c / (DKP / 8), col = (c % (DKP / 8)) * 8;
                 const unsigned off = col < dk ? ((tok0 + row) * (unsigned)dk + col) * (unsigned)sizeof(T) : kOob;
                 xr[u] = buf_load16(xb, need_x ? off : kOob);
                 yr[u] = buf_load16(yb, valid ? off : kOob);
             }
-            const int row = tid / 8, col = (tid % 8) * 8;
-            const unsigned off = (col0 + col < dv) ? ((tok0 + row) * (unsigned)dv + col0 + col) * (unsigned)sizeof(T) : kOob;
-            zr = buf_load16(zb, valid ? off : kOob);
+#pragma unroll
+            for (int u = 0; u < ZC; ++u) {
+                const int row = tid / 8 + (NL / 8) * u, col = (tid % 8) * 8;
+                const unsigned off = (col0 + col < dv) ? ((tok0 + row) * (unsigned)dv + col0 + col) * (unsigned)sizeof(T) : kOob;
+                zr[u] = buf_load16(zb, valid ? off : kOob);
+            }
             return;
         }
         const unsigned tok0 = valid ? (unsigned)(t * 64) : 0u;
@@ -198,21 +215,56 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepArgs a) {
             xr[u] = buf_load16(xb, lane_row < rows_x - u * CROWS ? lane_x : kOob, tk * xts * (unsigned)sizeof(T));
             yr[u] = buf_load16(yb, lane_row < rows - u * CROWS ? lane_y : kOob, tk * yts * (unsigned)sizeof(T));
         }
-        zr = buf_load16(zb, lane_zrow < rows ? lane_z : kOob, tok0 * zts * (unsigned)sizeof(T));
+#pragma unroll
+        for (int u = 0; u < ZC; ++u) {
+            const unsigned tk = u * (NL / 8) < rows ? tok0 + u * (NL / 8) : 0u;
+            zr[u] = buf_load16(zb, lane_zrow < rows - u * (NL / 8) ? lane_z : kOob, tk * zts * (unsigned)sizeof(T));
+        }
     };
     const unsigned lane_stage_xy = ((tid / (DKP / 8)) * XS + (tid % (DKP / 8)) * 8) * E;
     const unsigned lane_stage_z = ((tid / 8) * ZS + (tid % 8) * 8) * E;
-    auto stage_block = [&](int buf, const u32x4 (&xr)[XC], const u32x4 (&yr)[XC], const u32x4& zr) {
+    // Publishes a fetched block in tile buffer `buf`.  The z slot of that buffer still holds the
+    // output tile of the block that used it last (walk index bout; the state waves leave their
+    // columns of `out` there, over the z columns they alone read): every thread first takes the 16
+    // bytes its z chunk is about to replace and, if `flush`, sends them to memory - eight lanes
+    // write one whole 128-byte row segment.  (Stored straight from the accumulators, each wave
+    // would write 32-byte pieces of every row, which the memory system handles far worse: 0.083
+    // against 0.048 ms for the output traffic alone at the headline shape.)
+    const unsigned lane_o = (col0 + (tid % 8) * 8 < dv) ? (lane_zrow * ots + col0 + (tid % 8) * 8) * (unsigned)sizeof(T) : kOob;
+    auto store_out = [&](int64_t bout, bool flush, const u32x4 (&o)[ZC]) {
+        const int64_t t = REVERSE ? nblk - 1 - bout : bout;
+#pragma unroll
+        for (int u = 0; u < ZC; ++u) {
+            if (DENSE) {
+                // rows >= n fall outside the buffer and are dropped by the hardware range check
+                const unsigned tok0 = (unsigned)(t * 64) + u * (NL / 8);
+                const int col = col0 + (tid % 8) * 8;
+                const unsigned off = col < dv ? ((tok0 + lane_zrow) * (unsigned)dv + col) * (unsigned)sizeof(T) : kOob;
+                buf_store16(ob, flush ? off : kOob, 0u, o[u]);
+            } else {
+                const unsigned tok0 = flush ? (unsigned)(t * 64) : 0u;
+                const int rows = flush ? (int)min(64u, nrows - tok0) : 0;
+                const unsigned tk = u * (NL / 8) < rows ? tok0 + u * (NL / 8) : 0u;
+                buf_store16(ob, lane_zrow < rows - u * (NL / 8) ? lane_o : kOob, tk * ots * (unsigned)sizeof(T), o[u]);
+            }
+        }
+    };
+    auto stage_block = [&](int buf, const u32x4 (&xr)[XC], const u32x4 (&yr)[XC], const u32x4 (&zr)[ZC], int64_t bout, bool flush) {
         const unsigned xd = opaque(buf * XYB + lane_stage_xy);
         const unsigned zd = opaque(ZBASE + buf * ZTB + lane_stage_z);
+        u32x4 o[ZC];
+#pragma unroll
+        for (int u = 0; u < ZC; ++u) o[u] = *reinterpret_cast<const u32x4*>(smem + zd + u * (NL / 8) * ZS * E);
 #pragma unroll
         for (int u = 0; u < XC; ++u) {
-            // chunk c = tid + 512 u lies (512 / (DKP / 8)) rows below chunk tid
-            constexpr unsigned ROWS = 512 / (DKP / 8);
+            // chunk c = tid + NL u lies (NL / (DKP / 8)) rows below chunk tid
+            constexpr unsigned ROWS = NL / (DKP / 8);
             *reinterpret_cast<u32x4*>(smem + xd + u * ROWS * XS * E) = xr[u];
             *reinterpret_cast<u32x4*>(smem + xd + YOFF + u * ROWS * XS * E) = yr[u];
         }
-        *reinterpret_cast<u32x4*>(smem + zd) = zr;
+        store_out(bout, flush, o);
+#pragma unroll
+        for (int u = 0; u < ZC; ++u) *reinterpret_cast<u32x4*>(smem + zd + u * (NL / 8) * ZS * E) = zr[u];
     };
 
     // Score waves: S^T tiles of this wave for the block in tile buffer `buf` -> masked, decayed
@@ -279,12 +331,14 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepArgs a) {
 
     // zero both P buffers once: tiles on the masked side of the diagonal are never written
     for (int c = tid; c < 2 * L::PT / 8; c += 512) reinterpret_cast<uint4*>(smem + PBASE)[c] = make_uint4(0, 0, 0, 0);
-    load_block(0, xrA, yrA, zrA);
-    load_block(1, xrB, yrB, zrB);
-    stage_block(0, xrA, yrA, zrA);
-    load_block(2, xrA, yrA, zrA);
-    stage_block(1, xrB, yrB, zrB);
-    load_block(3, xrB, yrB, zrB);
+    if (loader) {
+        load_block(0, xrA, yrA, zrA);
+        load_block(1, xrB, yrB, zrB);
+        stage_block(0, xrA, yrA, zrA, 0, false);
+        load_block(2, xrA, yrA, zrA);
+        stage_block(1, xrB, yrB, zrB, 0, false);
+        load_block(3, xrB, yrB, zrB);
+    }
     __syncthreads();
     if (!state_role && it_first == 0) score_block(0, 0);
     __syncthreads();
@@ -295,21 +349,25 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepArgs a) {
     const unsigned lane_yt = ((8 * g + (r >> 2)) * XS + 4 * (r & 3)) * E;
     const unsigned lane_zt = ((8 * g + (r >> 2)) * ZS + 16 * w + 4 * (r & 3)) * E;
     const unsigned lane_pr = (r * PS + 8 * g) * E;
+    const unsigned lane_ow = (r * ZS + 16 * w + 4 * g) * E;  // out[i = r][16 w + 4 g ..] within 16 rows
 
     // One iteration.  `xr, yr, zr` hold block it+2 on entry and block it+4 on exit.
-    auto iteration = [&](const int64_t it, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4& zr) {
+    auto iteration = [&](auto role, const int64_t it, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4 (&zr)[ZC]) __attribute__((always_inline)) {
+        constexpr bool STATE = decltype(role)::value;
         const int64_t t = REVERSE ? nblk - 1 - it : it;
         const bool have_next = it + 1 < it_end;
         const bool warm = it < it_first;  // warm-up block: state update only
         const int bcur = (int)((unsigned)it % 3u);
         const int bnext = bcur == 2 ? 0 : bcur + 1;
         const int bstage = bnext == 2 ? 0 : bnext + 1;
-        // publish block it+2 (its buffer was last read in iteration it-1) and refill the
-        // registers with block it+4
-        stage_block(bstage, xr, yr, zr);
-        load_block(it + 4, xr, yr, zr);
+        // publish block it+2 (its buffer was last read in iteration it-1, whose output tile it
+        // still holds) and refill the registers with block it+4
+        if (NL == 512 || !STATE) {
+            stage_block(bstage, xr, yr, zr, it - 1, it > it_first);
+            load_block(it + 4, xr, yr, zr);
+        }
 
-        if (!state_role) {
+        if constexpr (!STATE) {
             if (have_next && it + 1 >= it_first) score_block(bnext, (int)((it + 1) & 1));
         } else if (cols_active) {
             const unsigned xq = opaque(bcur * XYB + lane_xq);
@@ -383,20 +441,15 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepArgs a) {
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                const int col = col0 + 16 * w + 4 * g;
+                // leave the tile in the z slot of this block, over this wave's own z columns (read
+                // above, and by no other wave); the next iteration's staging sends it to memory
+                const unsigned oq = opaque(ZBASE + bcur * ZTB + lane_ow);
 #pragma unroll
                 for (int i4 = 0; i4 < 4; ++i4) {
-                    const unsigned tok = (unsigned)(t * 64) + 16 * i4;  // wave-uniform first token of the tile
                     V4 o;
 #pragma unroll
                     for (int v = 0; v < 4; ++v) o[v] = (T)oacc[i4][v];
-                    if (DENSE) {
-                        const unsigned off = col < dv ? ((tok + r) * (unsigned)dv + col) * (unsigned)sizeof(T) : kOob;
-                        buf_store8(ob, off, __builtin_bit_cast(u32x2, o));
-                    } else {
-                        const unsigned off = (col < dv && tok + r < nrows) ? (r * ots + col) * (unsigned)sizeof(T) : kOob;
-                        buf_store8(ob, off, tok < nrows ? tok * ots * (unsigned)sizeof(T) : 0u, __builtin_bit_cast(u32x2, o));
-                    }
+                    *reinterpret_cast<V4*>(smem + oq + 16 * i4 * ZS * E) = o;
                 }
             }
             if (have_next) {
@@ -433,12 +486,26 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepArgs a) {
     };
     // Both halves of the unrolled loop always run, so the two register sets are refilled in the
     // same order on every path and the wait before staging one set leaves the other in flight.
-    int64_t it = 0;
-    for (; it + 1 < it_end; it += 2) {
-        iteration(it, xrA, yrA, zrA);
-        iteration(it + 1, xrB, yrB, zrB);
+    // The two kinds of waves run separate copies of the loop (one barrier per iteration in each),
+    // so that neither carries the other's registers.
+    auto walk = [&](auto role) __attribute__((always_inline)) {
+        int64_t it = 0;
+        for (; it + 1 < it_end; it += 2) {
+            iteration(role, it, xrA, yrA, zrA);
+            iteration(role, it + 1, xrB, yrB, zrB);
+        }
+        if (it < it_end) iteration(role, it, xrA, yrA, zrA);
+    };
+    if (state_role) walk(std::true_type{});
+    else walk(std::false_type{});
+    // the last block's output tile is still in its z slot
+    if (it_end > it_first && (NL == 512 || loader)) {
+        const unsigned zd = ZBASE + (unsigned)((it_end - 1) % 3) * ZTB + lane_stage_z;
+        u32x4 o[ZC];
+#pragma unroll
+        for (int u = 0; u < ZC; ++u) o[u] = *reinterpret_cast<const u32x4*>(smem + zd + u * (NL / 8) * ZS * E);
+        store_out(it_end - 1, true, o);
     }
-    if (it < it_end) iteration(it, xrA, yrA, zrA);
 }
 
 template <typename T, int DKP, bool REVERSE, bool DECAY, bool DENSE>
