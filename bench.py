@@ -173,7 +173,7 @@ def main():
         "frac": round(k_bytes / (k_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
         # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE (x2.0) + WRITE_SIZE (x1.0), see
         # profiles/la_sweep_pipe_kernel_b4_h32_n8192_d128_bf16.md; bench.py cannot read counters itself
-        "traffic": 1.0739e9,
+        "traffic": 1.0747e9,
         "traffic_unit": "bytes/launch (rocprofv3 counters, committed profile)",
         "algorithmic_bytes": k_bytes,
         "launch_ms": round(k_ms, 4),
