@@ -247,6 +247,27 @@ def test_sequence_chunking_is_exact(b, h, n, d, e, monkeypatch):
     check(outs[None], want, torch.bfloat16, "chunked %s" % ((b, h, n, d, e),))
 
 
+@pytest.mark.parametrize("chunks", ["2", "5"])
+def test_chunked_walk_on_projection_layout(chunks, monkeypatch):
+    """Chunked walk and token-major tensors together (ragged n, e off the 64 grid): the output tile of
+    every chunk's last block and the rows beyond n are the cases the write-back path has to get right."""
+    b, h, n, d, e = 1, 3, 1237, 128, 72
+    g = torch.Generator().manual_seed(23)
+    q, k = ((torch.randn(b, n, h, d, generator=g) * 0.7).bfloat16().to(DEV).transpose(1, 2) for _ in range(2))
+    v, do = (torch.randn(b, n, h, e, generator=g).bfloat16().to(DEV).transpose(1, 2) for _ in range(2))
+    s = _build_slope_tensor(h)
+    monkeypatch.setenv("LA_SWEEP_CHUNKS", chunks)
+    got = run_hip(q.detach(), k.detach(), v.detach(), s, do)  # fresh leaves for every call
+    got_plain = run_hip(q.contiguous(), k.contiguous(), v.contiguous(), s, do.contiguous())
+    monkeypatch.setenv("LA_SWEEP_CHUNKS", "1")
+    got_one = run_hip(q.detach(), k.detach(), v.detach(), s, do)
+    monkeypatch.delenv("LA_SWEEP_CHUNKS", raising=False)
+    for a, c, one in zip(got, got_plain, got_one):
+        assert torch.equal(a, c) and torch.equal(a, one)
+    want = oracle.linear_attn_fwd_bwd(q.cpu(), k.cpu(), v.cpu(), s, do.cpu(), torch.float32)
+    check(got, want, torch.bfloat16, "chunked token-major")
+
+
 def test_deterministic():
     q, k, v, do = make_inputs(2, 8, 1000, 128, 128, torch.bfloat16, 1.0)
     s = _build_slope_tensor(8)
