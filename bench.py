@@ -165,7 +165,7 @@ def main():
     k_bytes = bytes_per_token(D, D, "fwd") * tokens
     k_flop = flops_per_token(D, D, "fwd") * tokens
     roofline = {
-        "kernel": "la_sweep_pipe_kernel<bf16, DKP=128, forward, decay> (one launch: O = sweep(Q,K,V); a step is 4 such launches)",
+        "kernel": "la_sweep_pipe_kernel<bf16, DKP=128, forward, decay> (one launch: O = sweep(Q,K,V); a step is this, the same for dQ, and one double launch for dK + dV)",
         "bound": "hbm",
         "achieved": round(k_bytes / (k_ms * 1e-3) / 1e9, 1),
         "peak": PEAK_HBM_GBS,
@@ -173,7 +173,7 @@ def main():
         "frac": round(k_bytes / (k_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
         # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE (x2.0) + WRITE_SIZE (x1.0), see
         # profiles/la_sweep_pipe_kernel_b4_h32_n8192_d128_bf16.md; bench.py cannot read counters itself
-        "traffic": 1.0747e9,
+        "traffic": 1.0741e9,
         "traffic_unit": "bytes/launch (rocprofv3 counters, committed profile)",
         "algorithmic_bytes": k_bytes,
         "launch_ms": round(k_ms, 4),

@@ -3,9 +3,10 @@
 #include "lightning_attn_hip.h"
 
 namespace la {
-int sweep(const void* x, const void* y, const void* z, void* out, const Layout& lx, const Layout& ly, const Layout& lz,
-          const Layout& lo, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
+int sweep(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
           bool reverse, hipStream_t st);
+int sweep2(const SweepIO& io0, const SweepIO& io1, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv,
+           int dtype, bool reverse, hipStream_t st);
 int sweep_f32(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
               int64_t n, int64_t dk, int64_t dv, bool reverse, hipStream_t st);
 
@@ -20,6 +21,10 @@ static bool is_dense(const Tensor& t, int64_t h, int64_t n, int64_t cols) {
     return t.l.ts == cols && t.l.hs == n * cols && t.l.bs == h * n * cols;
 }
 
+static SweepIO io(const Tensor& x, const Tensor& y, const Tensor& z, const Tensor& out) {
+    return SweepIO{x.p, y.p, z.p, const_cast<void*>(out.p), x.l, y.l, z.l, out.l};
+}
+
 // one directional sweep at the element type named by dtype
 static int run(const Tensor& x, const Tensor& y, const Tensor& z, const Tensor& out, const float* s, int64_t bh, int64_t h,
                int64_t n, int64_t dk, int64_t dv, int dtype, bool reverse, hipStream_t st) {
@@ -29,7 +34,7 @@ static int run(const Tensor& x, const Tensor& y, const Tensor& z, const Tensor& 
             return LA_E_UNSUPPORTED;
         return sweep_f32(x.p, y.p, z.p, const_cast<void*>(out.p), s, bh, h, n, dk, dv, reverse, st);
     }
-    return sweep(x.p, y.p, z.p, const_cast<void*>(out.p), x.l, y.l, z.l, out.l, s, bh, h, n, dk, dv, dtype, reverse, st);
+    return sweep(io(x, y, z, out), s, bh, h, n, dk, dv, dtype, reverse, st);
 }
 
 static inline bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -85,10 +90,12 @@ static int bwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s
     // dQ_i = sum_{j<=i} lam^(i-j) (dO_i . v_j) k_j
     rc = run(dout, v, k, dq, s, b * h, h, n, e, d, dtype, false, st);
     if (rc != LA_OK) return rc;
-    // dK_j = sum_{i>=j} lam^(i-j) (v_j . dO_i) q_i
+    // dK_j = sum_{i>=j} lam^(i-j) (v_j . dO_i) q_i   and   dV_j = sum_{i>=j} lam^(i-j) (k_j . q_i) dO_i
+    // have the same shape when d == e: one launch, in which they share the reads of dO and q
+    if (d == e && dtype != LA_FP32)
+        return sweep2(io(v, dout, q, dk), io(k, q, dout, dv), s, b * h, h, n, d, e, dtype, true, st);
     rc = run(v, dout, q, dk, s, b * h, h, n, e, d, dtype, true, st);
     if (rc != LA_OK) return rc;
-    // dV_j = sum_{i>=j} lam^(i-j) (k_j . q_i) dO_i
     return run(k, q, dout, dv, s, b * h, h, n, d, e, dtype, true, st);
 }
 }  // namespace la

@@ -489,7 +489,7 @@ static int launch_dir(const SweepArgs& a, hipStream_t st) {
 // rebuild their incoming state themselves.  A warm-up block costs about half a full block, so
 // chunk lengths shrink geometrically (len_c ~ (1 - rho)^c, rho = 0.5) to make all workgroups
 // finish together.  LA_SWEEP_CHUNKS=<C> overrides the count.
-static void choose_chunks(SweepArgs& a) {
+static void choose_chunks(SweepArgs& a, int nprod = 1) {
     const char* env = getenv("LA_SWEEP_CHUNKS");  // read per call so that tests can vary it
     const int forced = env ? atoi(env) : 0;
     static const int cus = [] {
@@ -498,7 +498,7 @@ static void choose_chunks(SweepArgs& a) {
         return n > 0 ? n : 256;
     }();
     const int64_t nblk = (a.n + 63) / 64;
-    const int64_t wgs = (int64_t)((a.bh + 7) / 8 * 8) * a.nslice;
+    const int64_t wgs = (int64_t)((a.bh + 7) / 8 * 8) * a.nslice * nprod;
     int64_t c = 1;
     if (forced > 0) c = forced;
     else if (wgs * 2 <= cus && nblk >= 8) {
@@ -528,20 +528,48 @@ static void choose_chunks(SweepArgs& a) {
     for (int i = (int)c + 1; i < 9; ++i) a.chunk_start[i] = (int)nblk;
 }
 
-// x,y: (b,h,n,dk)  z,out: (b,h,n,dv), each with its own batch / head / token strides
-int sweep(const void* x, const void* y, const void* z, void* out, const Layout& lx, const Layout& ly, const Layout& lz,
-          const Layout& lo, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
-          bool reverse, hipStream_t st) {
+static SweepArgs make_args(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv) {
     SweepArgs a;
-    a.x = x; a.y = y; a.z = z; a.out = out; a.s = s;
-    a.lx = lx; a.ly = ly; a.lz = lz; a.lo = lo;
+    a.x = io.x; a.y = io.y; a.z = io.z; a.out = io.out; a.s = s;
+    a.lx = io.lx; a.ly = io.ly; a.lz = io.lz; a.lo = io.lo;
     a.n = n; a.dk = (int)dk; a.dv = (int)dv; a.h = (int)h; a.bh = (int)bh;
     a.nslice = (int)((dv + 63) / 64);
-    choose_chunks(a);
-    if (dk <= 128) return sweep_pipe(a, dtype, reverse, st);  // pipelined kernel, la_sweep_pipe.hip
+    return a;
+}
+
+static int launch_classic(const SweepArgs& a, int dtype, bool reverse, hipStream_t st) {
     if (dtype == LA_BF16) return reverse ? launch_dir<__bf16, true>(a, st) : launch_dir<__bf16, false>(a, st);
     if (dtype == LA_FP16) return reverse ? launch_dir<_Float16, true>(a, st) : launch_dir<_Float16, false>(a, st);
     return LA_E_UNSUPPORTED;
+}
+
+// x,y: (b,h,n,dk)  z,out: (b,h,n,dv), each with its own batch / head / token strides
+int sweep(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
+          bool reverse, hipStream_t st) {
+    SweepPair p;
+    p.nprod = 1;
+    p.a[0] = make_args(io, s, bh, h, n, dk, dv);
+    choose_chunks(p.a[0]);
+    p.a[1] = p.a[0];
+    if (dk <= 128) return sweep_pipe(p, dtype, reverse, st);  // pipelined kernel, la_sweep_pipe.hip
+    return launch_classic(p.a[0], dtype, reverse, st);
+}
+
+// Two sweeps of the same shape and direction; one launch where the pipelined kernel applies.
+int sweep2(const SweepIO& io0, const SweepIO& io1, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv,
+           int dtype, bool reverse, hipStream_t st) {
+    if (dk > 128 || getenv("LA_SWEEP_UNPAIRED")) {
+        const int rc = sweep(io0, s, bh, h, n, dk, dv, dtype, reverse, st);
+        return rc != LA_OK ? rc : sweep(io1, s, bh, h, n, dk, dv, dtype, reverse, st);
+    }
+    SweepPair p;
+    p.nprod = 2;
+    p.a[0] = make_args(io0, s, bh, h, n, dk, dv);
+    choose_chunks(p.a[0], 2);
+    p.a[1] = make_args(io1, s, bh, h, n, dk, dv);
+    p.a[1].nchunk = p.a[0].nchunk;
+    for (int i = 0; i < 9; ++i) p.a[1].chunk_start[i] = p.a[0].chunk_start[i];
+    return sweep_pipe(p, dtype, reverse, st);
 }
 
 }  // namespace la

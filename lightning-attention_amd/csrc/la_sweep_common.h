@@ -84,7 +84,24 @@ __device__ __constant__ const TileDeal kDeal[4] = {
     {0, 0, -1, -1, -1},
 };
 
+// Operands of one sweep: x, y (b, h, n, dk), z, out (b, h, n, dv), each with its own layout.
+struct SweepIO {
+    const void *x, *y, *z;
+    void* out;
+    Layout lx, ly, lz, lo;
+};
+
+// One launch of the pipelined kernel can carry two sweeps of the same shape, direction and layout
+// kind (dK and dV of the backward pass when d == e).  Their workgroups for one (batch, head) sit
+// next to each other on one XCD and walk the sequence in step, so the tensors the two sweeps have in
+// common (dO and Q) come from memory once and from that XCD's L2 the second time.
+struct SweepPair {
+    SweepArgs a[2];
+    int nprod;  // 1 or 2 sweeps; a[1] is unused when 1
+};
+
 // Launches the single-barrier pipelined kernel (feature dim up to 128); defined in la_sweep_pipe.hip.
-int sweep_pipe(const SweepArgs& a, int dtype, bool reverse, hipStream_t st);
+// n, dk, dv, h, bh, nslice and the chunking must agree between the two sweeps of a pair.
+int sweep_pipe(const SweepPair& p, int dtype, bool reverse, hipStream_t st);
 
 }  // namespace la

@@ -48,7 +48,7 @@ struct PipeLds {
 // DENSE: all four tensors are plain (b, h, n, d) arrays; their rows then take a shorter addressing path
 // (see load_block).
 template <typename T, int DKP, bool REVERSE, bool DECAY, bool DENSE>
-__global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepArgs a) {
+__global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
     typedef Mma<T> M;
     typedef typename M::V8 V8;
     typedef typename M::V4 V4;
@@ -84,10 +84,14 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepArgs a) {
     // Workgroups are dealt round-robin to the 8 XCDs by linear id; keep the
     // column slices of one head on one XCD so their x / y re-reads share an L2.
     const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-    const int per_unit = a.nslice * a.nchunk;
+    const int nslice = pair.a[0].nslice, nprod = pair.nprod;
+    const int per_unit = nslice * pair.a[0].nchunk * nprod;
     const int unit = xcd + 8 * (local / per_unit);
-    const int slice = (local % per_unit) % a.nslice;
-    const int chunk = (local % per_unit) / a.nslice;
+    const int sub = local % per_unit;
+    // the sweeps of a pair alternate fastest, then the column slices, then the sequence chunks
+    const SweepArgs& a = pair.a[sub % nprod];
+    const int slice = (sub / nprod) % nslice;
+    const int chunk = sub / (nprod * nslice);
     if (unit >= a.bh) return;
 
     const int tid = threadIdx.x;
@@ -509,7 +513,8 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepArgs a) {
 }
 
 template <typename T, int DKP, bool REVERSE, bool DECAY, bool DENSE>
-static int launch_one(const SweepArgs& a, hipStream_t st) {
+static int launch_one(const SweepPair& pair, hipStream_t st) {
+    const SweepArgs& a = pair.a[0];
     constexpr size_t lds = PipeLds<DKP>::bytes(sizeof(T));
     static_assert(lds <= 160 * 1024, "LDS budget");
     auto kern = la_sweep_pipe_kernel<T, DKP, REVERSE, DECAY, DENSE>;
@@ -519,8 +524,8 @@ static int launch_one(const SweepArgs& a, hipStream_t st) {
         if (e != hipSuccess) return (int)e;
     }
     const int units8 = (a.bh + 7) / 8 * 8;
-    const unsigned grid = (unsigned)(units8 * a.nslice * a.nchunk);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, st, a);
+    const unsigned grid = (unsigned)(units8 * a.nslice * a.nchunk * pair.nprod);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, st, pair);
     return (int)hipGetLastError();
 }
 
@@ -529,11 +534,16 @@ static bool plain(const Layout& l, int64_t h, int64_t n, int64_t cols) {
 }
 
 template <typename T, bool REVERSE>
-static int launch_dir(const SweepArgs& a, hipStream_t st) {
+static int launch_dir(const SweepPair& pair, hipStream_t st) {
+    const SweepArgs& a = pair.a[0];
     const bool decay = a.s != nullptr;
-    const bool dense = plain(a.lx, a.h, a.n, a.dk) && plain(a.ly, a.h, a.n, a.dk) && plain(a.lz, a.h, a.n, a.dv) &&
-                       plain(a.lo, a.h, a.n, a.dv);
-#define LA_GO2(DKP, DENSE) (decay ? launch_one<T, DKP, REVERSE, true, DENSE>(a, st) : launch_one<T, DKP, REVERSE, false, DENSE>(a, st))
+    bool dense = true;
+    for (int i = 0; i < pair.nprod; ++i) {
+        const SweepArgs& c = pair.a[i];
+        dense = dense && plain(c.lx, c.h, c.n, c.dk) && plain(c.ly, c.h, c.n, c.dk) && plain(c.lz, c.h, c.n, c.dv) &&
+                plain(c.lo, c.h, c.n, c.dv);
+    }
+#define LA_GO2(DKP, DENSE) (decay ? launch_one<T, DKP, REVERSE, true, DENSE>(pair, st) : launch_one<T, DKP, REVERSE, false, DENSE>(pair, st))
 #define LA_GO(DKP) (dense ? LA_GO2(DKP, true) : LA_GO2(DKP, false))
     if (a.dk <= 64) return LA_GO(64);
     return LA_GO(128);
@@ -541,10 +551,10 @@ static int launch_dir(const SweepArgs& a, hipStream_t st) {
 #undef LA_GO2
 }
 
-int sweep_pipe(const SweepArgs& a, int dtype, bool reverse, hipStream_t st) {
-    if (a.dk > 128) return LA_E_UNSUPPORTED;
-    if (dtype == LA_BF16) return reverse ? launch_dir<__bf16, true>(a, st) : launch_dir<__bf16, false>(a, st);
-    if (dtype == LA_FP16) return reverse ? launch_dir<_Float16, true>(a, st) : launch_dir<_Float16, false>(a, st);
+int sweep_pipe(const SweepPair& p, int dtype, bool reverse, hipStream_t st) {
+    if (p.a[0].dk > 128 || p.nprod < 1 || p.nprod > 2) return LA_E_UNSUPPORTED;
+    if (dtype == LA_BF16) return reverse ? launch_dir<__bf16, true>(p, st) : launch_dir<__bf16, false>(p, st);
+    if (dtype == LA_FP16) return reverse ? launch_dir<_Float16, true>(p, st) : launch_dir<_Float16, false>(p, st);
     return LA_E_UNSUPPORTED;
 }
 
