@@ -46,7 +46,7 @@ struct SweepLds {
 };
 
 template <typename T, int DKP, bool REVERSE, bool DECAY>
-__global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
+__global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepPair pair) {
     typedef Mma<T> M;
     typedef typename M::V8 V8;
     typedef typename M::V4 V4;
@@ -63,10 +63,14 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
     // Workgroups are dealt round-robin to the 8 XCDs by linear id; keep the
     // column slices of one head on one XCD so their x / y re-reads share an L2.
     const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-    const int per_unit = a.nslice * a.nchunk;
+    const int nslice = pair.a[0].nslice, nprod = pair.nprod;
+    const int per_unit = nslice * pair.a[0].nchunk * nprod;
     const int unit = xcd + 8 * (local / per_unit);
-    const int slice = (local % per_unit) % a.nslice;
-    const int chunk = (local % per_unit) / a.nslice;
+    const int sub = local % per_unit;
+    // the sweeps of a pair alternate fastest, then the column slices, then the sequence chunks
+    const SweepArgs& a = pair.a[sub % nprod];
+    const int slice = (sub / nprod) % nslice;
+    const int chunk = sub / (nprod * nslice);
     if (unit >= a.bh) return;
 
     const int tid = threadIdx.x;
@@ -460,7 +464,8 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepArgs a) {
 }
 
 template <typename T, int DKP, bool REVERSE, bool DECAY>
-static int launch_one(const SweepArgs& a, hipStream_t st) {
+static int launch_one(const SweepPair& pair, hipStream_t st) {
+    const SweepArgs& a = pair.a[0];
     constexpr size_t lds = SweepLds<DKP>::bytes(sizeof(T));
     static_assert(lds <= 160 * 1024, "LDS budget");
     auto kern = la_sweep_kernel<T, DKP, REVERSE, DECAY>;
@@ -470,15 +475,16 @@ static int launch_one(const SweepArgs& a, hipStream_t st) {
         if (e != hipSuccess) return (int)e;
     }
     const int units8 = (a.bh + 7) / 8 * 8;
-    const unsigned grid = (unsigned)(units8 * a.nslice * a.nchunk);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, st, a);
+    const unsigned grid = (unsigned)(units8 * a.nslice * a.nchunk * pair.nprod);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, st, pair);
     return (int)hipGetLastError();
 }
 
 template <typename T, bool REVERSE>
-static int launch_dir(const SweepArgs& a, hipStream_t st) {
+static int launch_dir(const SweepPair& pair, hipStream_t st) {
+    const SweepArgs& a = pair.a[0];
     const bool decay = a.s != nullptr;
-#define LA_GO(DKP) (decay ? launch_one<T, DKP, REVERSE, true>(a, st) : launch_one<T, DKP, REVERSE, false>(a, st))
+#define LA_GO(DKP) (decay ? launch_one<T, DKP, REVERSE, true>(pair, st) : launch_one<T, DKP, REVERSE, false>(pair, st))
     if (a.dk <= 192) return LA_GO(192);
     return LA_GO(256);
 #undef LA_GO
@@ -537,9 +543,9 @@ static SweepArgs make_args(const SweepIO& io, const float* s, int64_t bh, int64_
     return a;
 }
 
-static int launch_classic(const SweepArgs& a, int dtype, bool reverse, hipStream_t st) {
-    if (dtype == LA_BF16) return reverse ? launch_dir<__bf16, true>(a, st) : launch_dir<__bf16, false>(a, st);
-    if (dtype == LA_FP16) return reverse ? launch_dir<_Float16, true>(a, st) : launch_dir<_Float16, false>(a, st);
+static int launch_classic(const SweepPair& p, int dtype, bool reverse, hipStream_t st) {
+    if (dtype == LA_BF16) return reverse ? launch_dir<__bf16, true>(p, st) : launch_dir<__bf16, false>(p, st);
+    if (dtype == LA_FP16) return reverse ? launch_dir<_Float16, true>(p, st) : launch_dir<_Float16, false>(p, st);
     return LA_E_UNSUPPORTED;
 }
 
@@ -552,13 +558,13 @@ int sweep(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, i
     choose_chunks(p.a[0]);
     p.a[1] = p.a[0];
     if (dk <= 128) return sweep_pipe(p, dtype, reverse, st);  // pipelined kernel, la_sweep_pipe.hip
-    return launch_classic(p.a[0], dtype, reverse, st);
+    return launch_classic(p, dtype, reverse, st);
 }
 
-// Two sweeps of the same shape and direction; one launch where the pipelined kernel applies.
+// Two sweeps of the same shape and direction in one launch.
 int sweep2(const SweepIO& io0, const SweepIO& io1, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv,
            int dtype, bool reverse, hipStream_t st) {
-    if (dk > 128 || getenv("LA_SWEEP_UNPAIRED")) {
+    if (getenv("LA_SWEEP_UNPAIRED")) {  // for measurements: two launches
         const int rc = sweep(io0, s, bh, h, n, dk, dv, dtype, reverse, st);
         return rc != LA_OK ? rc : sweep(io1, s, bh, h, n, dk, dv, dtype, reverse, st);
     }
@@ -569,7 +575,8 @@ int sweep2(const SweepIO& io0, const SweepIO& io1, const float* s, int64_t bh, i
     p.a[1] = make_args(io1, s, bh, h, n, dk, dv);
     p.a[1].nchunk = p.a[0].nchunk;
     for (int i = 0; i < 9; ++i) p.a[1].chunk_start[i] = p.a[0].chunk_start[i];
-    return sweep_pipe(p, dtype, reverse, st);
+    if (dk <= 128) return sweep_pipe(p, dtype, reverse, st);
+    return launch_classic(p, dtype, reverse, st);
 }
 
 }  // namespace la
