@@ -268,6 +268,21 @@ def test_chunked_walk_on_projection_layout(chunks, monkeypatch):
     check(got, want, torch.bfloat16, "chunked token-major")
 
 
+@pytest.mark.parametrize("b, h, n, d", [(2, 4, 1000, 128), (1, 3, 777, 64), (1, 2, 500, 192), (1, 2, 300, 256)])
+def test_paired_backward_launch_matches_separate_launches(b, h, n, d, monkeypatch):
+    """With d == e the dK and dV sweeps travel in one launch (their workgroups share the reads of dO
+    and q); LA_SWEEP_UNPAIRED=1 launches them one after the other.  Same numbers, bit for bit."""
+    q, k, v, do = make_inputs(b, h, n, d, d, torch.bfloat16, 1.0, seed=d + n)
+    s = _build_slope_tensor(h)
+    monkeypatch.delenv("LA_SWEEP_UNPAIRED", raising=False)
+    paired = run_hip(q, k, v, s, do)
+    monkeypatch.setenv("LA_SWEEP_UNPAIRED", "1")
+    separate = run_hip(q, k, v, s, do)
+    monkeypatch.delenv("LA_SWEEP_UNPAIRED", raising=False)
+    for a, c in zip(paired, separate):
+        assert torch.equal(a, c)
+
+
 def test_deterministic():
     q, k, v, do = make_inputs(2, 8, 1000, 128, 128, torch.bfloat16, 1.0)
     s = _build_slope_tensor(8)
