@@ -385,31 +385,57 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
             for (int ks = 0; ks < 2; ++ks) {
                 zf[ks] = cat<V8, V4>(ldt(zq + 32 * ks * ZS * E), ldt(zq + (32 * ks + 4) * ZS * E));
             }
+            // y^T fragments of the state update, fetched in two halves: the first while the output
+            // of this block is finished, the second while the first is multiplied
+            V8 ay[KT][2];
+            auto read_ay = [&](int kt0, int kt1) {
+#pragma unroll
+                for (int kt = kt0; kt < kt1; ++kt) {
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks) {
+                        const unsigned py = yq + (32 * ks * XS + 16 * kt) * E;
+                        ay[kt][ks] = cat<V8, V4>(ldt(py), ldt(py + 4 * XS * E));
+                    }
+                }
+            };
+            constexpr int KH = KT / 2;
             if (!warm) {
                 // out^T[c][i] = Lout[i] * sum_k state[k][c] x[i][k]  +  sum_j z[j][c] P[i][j]
-                // The x fragments of contraction step ks+1 (and, at the end, the P fragments) are
-                // read while the MFMAs of step ks run.
-                auto read_x = [&](int ks, V8 (&bx)[4]) {
+                // All x fragments are requested up front: LDS answers in order, so the MFMAs of
+                // contraction step ks start as soon as its own fragments are there while the later
+                // ones are still on their way (one round trip for the whole product instead of one
+                // per step).
+                V8 bx[KS][4];
+                V8 bp[4][2];
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
                     for (int i4 = 0; i4 < 4; ++i4) {
                         // 8-byte reads from unrelated base registers (one per contraction step and
                         // half): fused in pairs into ds_read2_b64 they would conflict on the LDS
                         // banks at this row stride
                         const unsigned lo = opaque(xq + 32 * ks * E), hi = opaque(xq + (32 * ks + 16) * E);
-                        bx[i4] = cat<V8, V4>(ld4(lo + 16 * i4 * XS * E), ld4(hi + 16 * i4 * XS * E));
+                        bx[ks][i4] = cat<V8, V4>(ld4(lo + 16 * i4 * XS * E), ld4(hi + 16 * i4 * XS * E));
                     }
-                };
-                V8 bx[2][4];
-                V8 bp[4][2];
-                read_x(0, bx[0]);
+                    __builtin_amdgcn_sched_barrier(0);  // (keeps the address registers of one step at a time)
+                }
+                __builtin_amdgcn_sched_barrier(0);
                 f32x4 oacc[4];
 #pragma unroll
                 for (int i4 = 0; i4 < 4; ++i4) oacc[i4] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    if (ks + 1 < KS) {
-                        read_x(ks + 1, bx[(ks + 1) & 1]);
-                    } else {
+                    V8 sb;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        sb[v] = M::cvt(st[2 * ks][v]);
+                        sb[4 + v] = M::cvt(st[2 * ks + 1][v]);
+                    }
+#pragma unroll
+                    for (int i4 = 0; i4 < 4; ++i4) oacc[i4] = M::mma(sb, bx[ks][i4], oacc[i4]);
+                    if (ks == (KS - 1) / 2) {
+                        // the P fragments follow once half of the x fragments have been used up
+                        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                         for (int i4 = 0; i4 < 4; ++i4) {
 #pragma unroll
@@ -418,18 +444,12 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
                                 if (need) bp[i4][k2] = ld8(pq + (16 * i4 * PS + 32 * k2) * E);
                             }
                         }
+                        __builtin_amdgcn_sched_barrier(0);
                     }
-                    V8 sb;
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        sb[v] = M::cvt(st[2 * ks][v]);
-                        sb[4 + v] = M::cvt(st[2 * ks + 1][v]);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int i4 = 0; i4 < 4; ++i4) oacc[i4] = M::mma(sb, bx[ks & 1][i4], oacc[i4]);
-                    __builtin_amdgcn_sched_barrier(0);
                 }
+                __builtin_amdgcn_sched_barrier(0);
+                if (have_next) read_ay(0, KH);
+                __builtin_amdgcn_sched_barrier(0);
                 if (DECAY) {
 #pragma unroll
                     for (int i4 = 0; i4 < 4; ++i4)
@@ -455,18 +475,12 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
                     for (int v = 0; v < 4; ++v) o[v] = (T)oacc[i4][v];
                     *reinterpret_cast<V4*>(smem + oq + 16 * i4 * ZS * E) = o;
                 }
+            } else if (have_next) {
+                read_ay(0, KH);
             }
             if (have_next) {
                 // state = lam^64 state + y^T (z * Lupd)
-                V8 ay[KT][2];
-#pragma unroll
-                for (int kt = 0; kt < KT; ++kt) {
-#pragma unroll
-                    for (int ks = 0; ks < 2; ++ks) {
-                        const unsigned py = yq + (32 * ks * XS + 16 * kt) * E;
-                        ay[kt][ks] = cat<V8, V4>(ldt(py), ldt(py + 4 * XS * E));
-                    }
-                }
+                read_ay(KH, KT);
                 __builtin_amdgcn_sched_barrier(0);
                 if (DECAY) {
 #pragma unroll
@@ -500,15 +514,24 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
         }
         if (it < it_end) iteration(role, it, xrA, yrA, zrA);
     };
-    if (state_role) walk(std::true_type{});
-    else walk(std::false_type{});
-    // the last block's output tile is still in its z slot
-    if (it_end > it_first && (NL == 512 || loader)) {
+    // the last block's output tile is still in its z slot when the walk ends
+    auto flush_last = [&]() {
+        if (it_end <= it_first) return;
         const unsigned zd = ZBASE + (unsigned)((it_end - 1) % 3) * ZTB + lane_stage_z;
         u32x4 o[ZC];
 #pragma unroll
         for (int u = 0; u < ZC; ++u) o[u] = *reinterpret_cast<const u32x4*>(smem + zd + u * (NL / 8) * ZS * E);
         store_out(it_end - 1, true, o);
+    };
+    if (state_role) {
+        // The state waves are the critical path and every SIMD holds one wave of each kind: when both
+        // have an instruction ready (right after the barrier all eight waves go for LDS), theirs goes first.
+        __builtin_amdgcn_s_setprio(1);
+        walk(std::true_type{});
+        if (NL == 512) flush_last();
+    } else {
+        walk(std::false_type{});
+        flush_last();
     }
 }
 
