@@ -56,12 +56,9 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
     constexpr int XS = L::XS, ZS = L::ZS, PS = L::PS;
     constexpr int KS = DKP / 32;  // 32-wide contraction steps over the feature dim
     constexpr int KT = DKP / 16;  // 16-row state tiles
-#ifndef LA_PIPE_LOADERS
-#define LA_PIPE_LOADERS 256
-#endif
     // Threads that fetch, publish and write back the tiles: the 256 of the score waves, which have
     // slack; the state waves' serial chain then holds no memory instructions at all.
-    constexpr int NL = LA_PIPE_LOADERS;
+    constexpr int NL = 256;
     constexpr int XC = 64 * (DKP / 8) / NL;  // 16-byte chunks per loader thread for an x / y tile
     constexpr int ZC = 512 / NL;             // ... and for the z slice / the output tile
     extern __shared__ __align__(16) unsigned char smem[];
@@ -169,7 +166,6 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
     const int64_t it_end = a.chunk_start[chunk + 1];
 
     u32x4 xrA[XC], yrA[XC], zrA[ZC], xrB[XC], yrB[XC], zrB[ZC];
-    const bool loader = tid < NL;
 
     // Per-lane byte offsets of this thread's first 16-byte chunk inside a 64-token block (out of
     // range where the chunk lies in the zero padding dk..DKP-1 or beyond dv).  Its further chunks
@@ -335,7 +331,7 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
 
     // zero both P buffers once: tiles on the masked side of the diagonal are never written
     for (int c = tid; c < 2 * L::PT / 8; c += 512) reinterpret_cast<uint4*>(smem + PBASE)[c] = make_uint4(0, 0, 0, 0);
-    if (loader) {
+    if (!state_role) {
         load_block(0, xrA, yrA, zrA);
         load_block(1, xrB, yrB, zrB);
         stage_block(0, xrA, yrA, zrA, 0, false);
@@ -366,12 +362,9 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
         const int bstage = bnext == 2 ? 0 : bnext + 1;
         // publish block it+2 (its buffer was last read in iteration it-1, whose output tile it
         // still holds) and refill the registers with block it+4
-        if (NL == 512 || !STATE) {
+        if constexpr (!STATE) {
             stage_block(bstage, xr, yr, zr, it - 1, it > it_first);
             load_block(it + 4, xr, yr, zr);
-        }
-
-        if constexpr (!STATE) {
             if (have_next && it + 1 >= it_first) score_block(bnext, (int)((it + 1) & 1));
         } else if (cols_active) {
             const unsigned xq = opaque(bcur * XYB + lane_xq);
@@ -385,20 +378,6 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
             for (int ks = 0; ks < 2; ++ks) {
                 zf[ks] = cat<V8, V4>(ldt(zq + 32 * ks * ZS * E), ldt(zq + (32 * ks + 4) * ZS * E));
             }
-            // y^T fragments of the state update, fetched in two halves: the first while the output
-            // of this block is finished, the second while the first is multiplied
-            V8 ay[KT][2];
-            auto read_ay = [&](int kt0, int kt1) {
-#pragma unroll
-                for (int kt = kt0; kt < kt1; ++kt) {
-#pragma unroll
-                    for (int ks = 0; ks < 2; ++ks) {
-                        const unsigned py = yq + (32 * ks * XS + 16 * kt) * E;
-                        ay[kt][ks] = cat<V8, V4>(ldt(py), ldt(py + 4 * XS * E));
-                    }
-                }
-            };
-            constexpr int KH = KT / 2;
             if (!warm) {
                 // out^T[c][i] = Lout[i] * sum_k state[k][c] x[i][k]  +  sum_j z[j][c] P[i][j]
                 // All x fragments are requested up front: LDS answers in order, so the MFMAs of
@@ -448,8 +427,6 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                if (have_next) read_ay(0, KH);
-                __builtin_amdgcn_sched_barrier(0);
                 if (DECAY) {
 #pragma unroll
                     for (int i4 = 0; i4 < 4; ++i4)
@@ -475,12 +452,18 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
                     for (int v = 0; v < 4; ++v) o[v] = (T)oacc[i4][v];
                     *reinterpret_cast<V4*>(smem + oq + 16 * i4 * ZS * E) = o;
                 }
-            } else if (have_next) {
-                read_ay(0, KH);
             }
             if (have_next) {
                 // state = lam^64 state + y^T (z * Lupd)
-                read_ay(KH, KT);
+                V8 ay[KT][2];
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks) {
+                        const unsigned py = yq + (32 * ks * XS + 16 * kt) * E;
+                        ay[kt][ks] = cat<V8, V4>(ldt(py), ldt(py + 4 * XS * E));
+                    }
+                }
                 __builtin_amdgcn_sched_barrier(0);
                 if (DECAY) {
 #pragma unroll
@@ -528,7 +511,6 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
         // have an instruction ready (right after the barrier all eight waves go for LDS), theirs goes first.
         __builtin_amdgcn_s_setprio(1);
         walk(std::true_type{});
-        if (NL == 512) flush_last();
     } else {
         walk(std::false_type{});
         flush_last();
