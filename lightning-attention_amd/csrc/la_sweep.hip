@@ -495,14 +495,19 @@ static int launch_dir(const SweepPair& pair, hipStream_t st) {
 // rebuild their incoming state themselves.  A warm-up block costs about half a full block, so
 // chunk lengths shrink geometrically (len_c ~ (1 - rho)^c, rho = 0.5) to make all workgroups
 // finish together.  LA_SWEEP_CHUNKS=<C> overrides the count.
-static void choose_chunks(SweepArgs& a, int nprod = 1) {
-    const char* env = getenv("LA_SWEEP_CHUNKS");  // read per call so that tests can vary it
-    const int forced = env ? atoi(env) : 0;
+static int num_cus() {
     static const int cus = [] {
         int dev = 0, n = 256;
         if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
         return n > 0 ? n : 256;
     }();
+    return cus;
+}
+
+static void choose_chunks(SweepArgs& a, int nprod = 1) {
+    const char* env = getenv("LA_SWEEP_CHUNKS");  // read per call so that tests can vary it
+    const int forced = env ? atoi(env) : 0;
+    const int cus = num_cus();
     const int64_t nblk = (a.n + 63) / 64;
     const int64_t wgs = (int64_t)((a.bh + 7) / 8 * 8) * a.nslice * nprod;
     int64_t c = 1;
@@ -534,6 +539,17 @@ static void choose_chunks(SweepArgs& a, int nprod = 1) {
     for (int i = (int)c + 1; i < 9; ++i) a.chunk_start[i] = (int)nblk;
 }
 
+// Where 128-column workgroups still fill the chip, the pipelined kernel gives each workgroup 128
+// columns of z / out instead of 64: the score tile and the x / y tiles are then produced once per
+// 128 output columns, and the power-limited kernel turns the saved work into time (dK + dV at the
+// headline shape: 0.31 against 0.415 ms).  LA_SWEEP_WIDE=0 / 1 overrides the choice.
+static bool wide_columns(int64_t bh, int64_t dk, int64_t dv, int nprod) {
+    if (dk > 128 || dv <= 64 || dv > 128) return false;
+    const char* env = getenv("LA_SWEEP_WIDE");
+    if (env) return atoi(env) != 0;
+    return (int64_t)((bh + 7) / 8 * 8) * nprod >= num_cus();
+}
+
 static SweepArgs make_args(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv) {
     SweepArgs a;
     a.x = io.x; a.y = io.y; a.z = io.z; a.out = io.out; a.s = s;
@@ -554,7 +570,9 @@ int sweep(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, i
           bool reverse, hipStream_t st) {
     SweepPair p;
     p.nprod = 1;
+    p.wide = wide_columns(bh, dk, dv, 1) ? 1 : 0;
     p.a[0] = make_args(io, s, bh, h, n, dk, dv);
+    if (p.wide) p.a[0].nslice = 1;
     choose_chunks(p.a[0]);
     p.a[1] = p.a[0];
     if (dk <= 128) return sweep_pipe(p, dtype, reverse, st);  // pipelined kernel, la_sweep_pipe.hip
@@ -571,8 +589,10 @@ int sweep2(const SweepIO& io0, const SweepIO& io1, const float* s, int64_t bh, i
     SweepPair p;
     p.nprod = 2;
     p.a[0] = make_args(io0, s, bh, h, n, dk, dv);
-    choose_chunks(p.a[0], 2);
     p.a[1] = make_args(io1, s, bh, h, n, dk, dv);
+    p.wide = wide_columns(bh, dk, dv, 2) ? 1 : 0;
+    if (p.wide) p.a[0].nslice = p.a[1].nslice = 1;
+    choose_chunks(p.a[0], 2);
     p.a[1].nchunk = p.a[0].nchunk;
     for (int i = 0; i < 9; ++i) p.a[1].chunk_start[i] = p.a[0].chunk_start[i];
     if (dk <= 128) return sweep_pipe(p, dtype, reverse, st);

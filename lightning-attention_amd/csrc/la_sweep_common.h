@@ -98,6 +98,7 @@ struct SweepIO {
 struct SweepPair {
     SweepArgs a[2];
     int nprod;  // 1 or 2 sweeps; a[1] is unused when 1
+    int wide;   // pipelined kernel only: a workgroup covers 128 instead of 64 columns of z / out
 };
 
 // Launches the single-barrier pipelined kernel (feature dim up to 128); defined in la_sweep_pipe.hip.

@@ -28,7 +28,8 @@
 
 namespace la {
 
-template <int DKP>
+// NH: 16-column accumulator slabs per state wave; a workgroup covers 64 NH columns of z / out.
+template <int DKP, int NH>
 struct PipeLds {
 #ifndef LA_PIPE_XPAD
 #define LA_PIPE_XPAD 16
@@ -37,22 +38,23 @@ struct PipeLds {
 #ifndef LA_PIPE_PPAD
 #define LA_PIPE_PPAD 8
 #endif
-    static constexpr int ZS = 64 + 8;             // row stride of the z slice
+    static constexpr int ZS = 64 * NH + 8;        // row stride of the z slice
+    static constexpr int NZ = NH == 1 ? 3 : 2;    // z / out slots (see the kernel)
     static constexpr int PS = 64 + LA_PIPE_PPAD;  // row stride of the P tile
     static constexpr int XY = 2 * 64 * XS;        // elements of one x + y buffer
     static constexpr int ZT = 64 * ZS;            // elements of one z buffer
     static constexpr int PT = 64 * PS;            // elements of one P buffer
-    static constexpr size_t bytes(size_t elt) { return (size_t)(3 * XY + 3 * ZT + 2 * PT) * elt; }
+    static constexpr size_t bytes(size_t elt) { return (size_t)(3 * XY + NZ * ZT + 2 * PT) * elt; }
 };
 
 // DENSE: all four tensors are plain (b, h, n, d) arrays; their rows then take a shorter addressing path
 // (see load_block).
-template <typename T, int DKP, bool REVERSE, bool DECAY, bool DENSE>
+template <typename T, int DKP, int NH, bool REVERSE, bool DECAY, bool DENSE>
 __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
     typedef Mma<T> M;
     typedef typename M::V8 V8;
     typedef typename M::V4 V4;
-    typedef PipeLds<DKP> L;
+    typedef PipeLds<DKP, NH> L;
     constexpr int XS = L::XS, ZS = L::ZS, PS = L::PS;
     constexpr int KS = DKP / 32;  // 32-wide contraction steps over the feature dim
     constexpr int KT = DKP / 16;  // 16-row state tiles
@@ -60,16 +62,24 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
     // slack; the state waves' serial chain then holds no memory instructions at all.
     constexpr int NL = 256;
     constexpr int XC = 64 * (DKP / 8) / NL;  // 16-byte chunks per loader thread for an x / y tile
-    constexpr int ZC = 512 / NL;             // ... and for the z slice / the output tile
+    constexpr int ZW = 64 * NH;              // columns of z / out per workgroup
+    constexpr int CPR = ZW / 8;              // 16-byte chunks per row of the z slice
+    constexpr int ZC = 64 * CPR / NL;        // chunks per loader thread for the z slice / the output tile
+    constexpr int ZROWS = NL / CPR;          // rows between two of them
+    constexpr int NZ = L::NZ;
+    // NH = 2: there is room for two z slots only, so the z slice of a block is published one
+    // iteration later than its x / y tiles (it is first needed one iteration later, too) and
+    // travels one register set behind them.
+    constexpr int ZLAG = NH - 1;
     extern __shared__ __align__(16) unsigned char smem[];
-    // LDS map in bytes: [3][x 64*XS | y 64*XS] tiles, [3][64*ZS] z tiles, [2][64*PS] P tiles.
+    // LDS map in bytes: [3][x 64*XS | y 64*XS] tiles, [NZ][64*ZS] z tiles, [2][64*PS] P tiles.
     // All LDS accesses below are written as (per-iteration base register) + (compile-time
     // constant), which the DS instructions take as register + immediate offset; the bases are
     // made opaque to the optimiser once per iteration so that it does not keep one address
     // register per access alive across the loop.
     constexpr unsigned E = (unsigned)sizeof(T);
     constexpr unsigned XYB = L::XY * E, ZTB = L::ZT * E, PTB = L::PT * E, YOFF = 64 * XS * E;
-    constexpr unsigned ZBASE = 3 * XYB, PBASE = ZBASE + 3 * ZTB;
+    constexpr unsigned ZBASE = 3 * XYB, PBASE = ZBASE + NZ * ZTB;
     auto opaque = [](unsigned v) {
         asm volatile("" : "+v"(v));
         return v;
@@ -105,8 +115,9 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
     const __amdgpu_buffer_rsrc_t ob = seq_rsrc<T>(a.out, a.lo, unit, a.h, n, dv);
     const unsigned xts = (unsigned)a.lx.ts, yts = (unsigned)a.ly.ts, zts = (unsigned)a.lz.ts, ots = (unsigned)a.lo.ts;
     const unsigned nrows = (unsigned)n;
-    const int col0 = slice * 64;
-    const bool cols_active = (col0 + 16 * w) < dv;
+    const int col0 = slice * ZW;
+    const int cbase = 16 * NH * w;  // first of this state wave's 16 NH columns within the slice
+    const bool cols_active = (col0 + cbase) < dv;
 
     float rate = 0.f;
     if (DECAY) rate = a.s[unit % a.h];
@@ -154,9 +165,7 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
         lamB = expf(-rate * 64.f);
     }
 
-    f32x4 st[KT];
-#pragma unroll
-    for (int kt = 0; kt < KT; ++kt) st[kt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    f32x4 st[NH][KT];  // the state; zeroed where the state waves start their walk
 
     const int64_t nblk = (n + 63) / 64;
     // Sequence chunking: this workgroup produces the blocks [it_first, it_end) of the walk.  It
@@ -175,14 +184,17 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
     const int lane_row = tid / (DKP / 8), lane_col = (tid % (DKP / 8)) * 8;
     const unsigned lane_x = lane_col < dk ? (lane_row * xts + lane_col) * (unsigned)sizeof(T) : kOob;
     const unsigned lane_y = lane_col < dk ? (lane_row * yts + lane_col) * (unsigned)sizeof(T) : kOob;
-    const int lane_zrow = tid / 8;
-    const unsigned lane_z = (col0 + (tid % 8) * 8 < dv) ? (lane_zrow * zts + col0 + (tid % 8) * 8) * (unsigned)sizeof(T) : kOob;
+    const int lane_zrow = tid / CPR, lane_zcol = col0 + (tid % CPR) * 8;
+    const unsigned lane_z = lane_zcol < dv ? (lane_zrow * zts + lane_zcol) * (unsigned)sizeof(T) : kOob;
     // Fetches block number b of the walk.  Blocks at or beyond it_end, and the x tile of warm-up
     // blocks, are fetched at the out-of-range offset: zeros, no memory traffic, and the loads are
     // issued unconditionally (no branches, no draining `s_waitcnt vmcnt(0)` at joins).
     auto load_block = [&](int64_t b, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4 (&zr)[ZC]) {
         const int64_t t = REVERSE ? nblk - 1 - b : b;
         const bool valid = b < it_end, need_x = valid && b >= it_first;
+        // the z slice that travels with this block's x / y tiles
+        const int64_t bz = b - ZLAG, tz = REVERSE ? nblk - 1 - bz : bz;
+        const bool validz = bz >= 0 && bz < it_end;
         if (DENSE) {
             // Plain tensors: one per-lane offset, rows >= n fall outside the buffer and the hardware
             // range check zeroes them.  Kept as its own code path because it is measurably faster
@@ -197,11 +209,12 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
                 xr[u] = buf_load16(xb, need_x ? off : kOob);
                 yr[u] = buf_load16(yb, valid ? off : kOob);
             }
+            const unsigned tokz = (unsigned)(tz * 64);
 #pragma unroll
             for (int u = 0; u < ZC; ++u) {
-                const int row = tid / 8 + (NL / 8) * u, col = (tid % 8) * 8;
-                const unsigned off = (col0 + col < dv) ? ((tok0 + row) * (unsigned)dv + col0 + col) * (unsigned)sizeof(T) : kOob;
-                zr[u] = buf_load16(zb, valid ? off : kOob);
+                const int row = lane_zrow + ZROWS * u;
+                const unsigned off = lane_zcol < dv ? ((tokz + row) * (unsigned)dv + lane_zcol) * (unsigned)sizeof(T) : kOob;
+                zr[u] = buf_load16(zb, validz ? off : kOob);
             }
             return;
         }
@@ -215,14 +228,16 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
             xr[u] = buf_load16(xb, lane_row < rows_x - u * CROWS ? lane_x : kOob, tk * xts * (unsigned)sizeof(T));
             yr[u] = buf_load16(yb, lane_row < rows - u * CROWS ? lane_y : kOob, tk * yts * (unsigned)sizeof(T));
         }
+        const unsigned tokz = validz ? (unsigned)(tz * 64) : 0u;
+        const int rowsz = validz ? (int)min(64u, nrows - tokz) : 0;
 #pragma unroll
         for (int u = 0; u < ZC; ++u) {
-            const unsigned tk = u * (NL / 8) < rows ? tok0 + u * (NL / 8) : 0u;
-            zr[u] = buf_load16(zb, lane_zrow < rows - u * (NL / 8) ? lane_z : kOob, tk * zts * (unsigned)sizeof(T));
+            const unsigned tk = u * ZROWS < rowsz ? tokz + u * ZROWS : 0u;
+            zr[u] = buf_load16(zb, lane_zrow < rowsz - u * ZROWS ? lane_z : kOob, tk * zts * (unsigned)sizeof(T));
         }
     };
     const unsigned lane_stage_xy = ((tid / (DKP / 8)) * XS + (tid % (DKP / 8)) * 8) * E;
-    const unsigned lane_stage_z = ((tid / 8) * ZS + (tid % 8) * 8) * E;
+    const unsigned lane_stage_z = (lane_zrow * ZS + (tid % CPR) * 8) * E;
     // Publishes a fetched block in tile buffer `buf`.  The z slot of that buffer still holds the
     // output tile of the block that used it last (walk index bout; the state waves leave their
     // columns of `out` there, over the z columns they alone read): every thread first takes the 16
@@ -230,31 +245,30 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
     // write one whole 128-byte row segment.  (Stored straight from the accumulators, each wave
     // would write 32-byte pieces of every row, which the memory system handles far worse: 0.083
     // against 0.048 ms for the output traffic alone at the headline shape.)
-    const unsigned lane_o = (col0 + (tid % 8) * 8 < dv) ? (lane_zrow * ots + col0 + (tid % 8) * 8) * (unsigned)sizeof(T) : kOob;
+    const unsigned lane_o = lane_zcol < dv ? (lane_zrow * ots + lane_zcol) * (unsigned)sizeof(T) : kOob;
     auto store_out = [&](int64_t bout, bool flush, const u32x4 (&o)[ZC]) {
         const int64_t t = REVERSE ? nblk - 1 - bout : bout;
 #pragma unroll
         for (int u = 0; u < ZC; ++u) {
             if (DENSE) {
                 // rows >= n fall outside the buffer and are dropped by the hardware range check
-                const unsigned tok0 = (unsigned)(t * 64) + u * (NL / 8);
-                const int col = col0 + (tid % 8) * 8;
-                const unsigned off = col < dv ? ((tok0 + lane_zrow) * (unsigned)dv + col) * (unsigned)sizeof(T) : kOob;
+                const unsigned tok0 = (unsigned)(t * 64) + u * ZROWS;
+                const unsigned off = lane_zcol < dv ? ((tok0 + lane_zrow) * (unsigned)dv + lane_zcol) * (unsigned)sizeof(T) : kOob;
                 buf_store16(ob, flush ? off : kOob, 0u, o[u]);
             } else {
                 const unsigned tok0 = flush ? (unsigned)(t * 64) : 0u;
                 const int rows = flush ? (int)min(64u, nrows - tok0) : 0;
-                const unsigned tk = u * (NL / 8) < rows ? tok0 + u * (NL / 8) : 0u;
-                buf_store16(ob, lane_zrow < rows - u * (NL / 8) ? lane_o : kOob, tk * ots * (unsigned)sizeof(T), o[u]);
+                const unsigned tk = u * ZROWS < rows ? tok0 + u * ZROWS : 0u;
+                buf_store16(ob, lane_zrow < rows - u * ZROWS ? lane_o : kOob, tk * ots * (unsigned)sizeof(T), o[u]);
             }
         }
     };
-    auto stage_block = [&](int buf, const u32x4 (&xr)[XC], const u32x4 (&yr)[XC], const u32x4 (&zr)[ZC], int64_t bout, bool flush) {
+    auto stage_block = [&](int buf, int zslot, const u32x4 (&xr)[XC], const u32x4 (&yr)[XC], const u32x4 (&zr)[ZC], int64_t bout, bool flush) {
         const unsigned xd = opaque(buf * XYB + lane_stage_xy);
-        const unsigned zd = opaque(ZBASE + buf * ZTB + lane_stage_z);
+        const unsigned zd = opaque(ZBASE + zslot * ZTB + lane_stage_z);
         u32x4 o[ZC];
 #pragma unroll
-        for (int u = 0; u < ZC; ++u) o[u] = *reinterpret_cast<const u32x4*>(smem + zd + u * (NL / 8) * ZS * E);
+        for (int u = 0; u < ZC; ++u) o[u] = *reinterpret_cast<const u32x4*>(smem + zd + u * ZROWS * ZS * E);
 #pragma unroll
         for (int u = 0; u < XC; ++u) {
             // chunk c = tid + NL u lies (NL / (DKP / 8)) rows below chunk tid
@@ -264,7 +278,7 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
         }
         store_out(bout, flush, o);
 #pragma unroll
-        for (int u = 0; u < ZC; ++u) *reinterpret_cast<u32x4*>(smem + zd + u * (NL / 8) * ZS * E) = zr[u];
+        for (int u = 0; u < ZC; ++u) *reinterpret_cast<u32x4*>(smem + zd + u * ZROWS * ZS * E) = zr[u];
     };
 
     // Score waves: S^T tiles of this wave for the block in tile buffer `buf` -> masked, decayed
@@ -331,25 +345,13 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
 
     // zero both P buffers once: tiles on the masked side of the diagonal are never written
     for (int c = tid; c < 2 * L::PT / 8; c += 512) reinterpret_cast<uint4*>(smem + PBASE)[c] = make_uint4(0, 0, 0, 0);
-    if (!state_role) {
-        load_block(0, xrA, yrA, zrA);
-        load_block(1, xrB, yrB, zrB);
-        stage_block(0, xrA, yrA, zrA, 0, false);
-        load_block(2, xrA, yrA, zrA);
-        stage_block(1, xrB, yrB, zrB, 0, false);
-        load_block(3, xrB, yrB, zrB);
-    }
-    __syncthreads();
-    if (!state_role && it_first == 0) score_block(0, 0);
-    __syncthreads();
-
     // state-wave lane offsets: x fragment halves (row r, columns 4g..), transposed reads of y and
     // of this wave's 16 z columns (row 8g + r/4, columns 4 (r%4)..), P fragments (row r, chunk g)
     const unsigned lane_xq = (r * XS + 4 * g) * E;
     const unsigned lane_yt = ((8 * g + (r >> 2)) * XS + 4 * (r & 3)) * E;
-    const unsigned lane_zt = ((8 * g + (r >> 2)) * ZS + 16 * w + 4 * (r & 3)) * E;
+    const unsigned lane_zt = ((8 * g + (r >> 2)) * ZS + cbase + 4 * (r & 3)) * E;
     const unsigned lane_pr = (r * PS + 8 * g) * E;
-    const unsigned lane_ow = (r * ZS + 16 * w + 4 * g) * E;  // out[i = r][16 w + 4 g ..] within 16 rows
+    const unsigned lane_ow = (r * ZS + cbase + 4 * g) * E;  // out[i = r][cbase + 4 g ..] within 16 rows
 
     // One iteration.  `xr, yr, zr` hold block it+2 on entry and block it+4 on exit.
     auto iteration = [&](auto role, const int64_t it, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4 (&zr)[ZC]) __attribute__((always_inline)) {
@@ -363,95 +365,113 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
         // publish block it+2 (its buffer was last read in iteration it-1, whose output tile it
         // still holds) and refill the registers with block it+4
         if constexpr (!STATE) {
-            stage_block(bstage, xr, yr, zr, it - 1, it > it_first);
+            stage_block(bstage, NH == 1 ? bstage : (int)((it + 1) & 1), xr, yr, zr, it - 1, it > it_first);
             load_block(it + 4, xr, yr, zr);
             if (have_next && it + 1 >= it_first) score_block(bnext, (int)((it + 1) & 1));
         } else if (cols_active) {
             const unsigned xq = opaque(bcur * XYB + lane_xq);
             const unsigned yq = opaque(bcur * XYB + YOFF + lane_yt);
-            const unsigned zq = opaque(ZBASE + bcur * ZTB + lane_zt);
+            const int zcur = NH == 1 ? bcur : (int)(it & 1);  // z / out slot of this block
+            const unsigned zq = opaque(ZBASE + zcur * ZTB + lane_zt);
             const unsigned pq = opaque(PBASE + (unsigned)(it & 1) * PTB + lane_pr);
-            // z^T fragments of this wave's 16 columns: A operand of the intra-block product and,
-            // scaled, B operand of the state update
-            V8 zf[2];
+            // z^T fragments of this wave's 16-column slabs: A operand of the intra-block product
+            // and, scaled, B operand of the state update
+            V8 zf[NH][2];
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                zf[ks] = cat<V8, V4>(ldt(zq + 32 * ks * ZS * E), ldt(zq + (32 * ks + 4) * ZS * E));
-            }
+            for (int h = 0; h < NH; ++h)
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks)
+                    zf[h][ks] = cat<V8, V4>(ldt(zq + (32 * ks * ZS + 16 * h) * E), ldt(zq + ((32 * ks + 4) * ZS + 16 * h) * E));
             if (!warm) {
                 // out^T[c][i] = Lout[i] * sum_k state[k][c] x[i][k]  +  sum_j z[j][c] P[i][j]
-                // All x fragments are requested up front: LDS answers in order, so the MFMAs of
-                // contraction step ks start as soon as its own fragments are there while the later
-                // ones are still on their way (one round trip for the whole product instead of one
-                // per step).
-                V8 bx[KS][4];
+                // One slab: all x fragments are requested up front; LDS answers in order, so the
+                // MFMAs of contraction step ks start as soon as its own fragments are there while
+                // the later ones are still on their way.  Two slabs: every fragment feeds both, and
+                // there are registers for one step of look-ahead only.
+                constexpr int NBX = NH == 1 ? KS : 2;
+                V8 bx[NBX][4];
                 V8 bp[4][2];
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
+                auto read_x = [&](int ks) {
 #pragma unroll
                     for (int i4 = 0; i4 < 4; ++i4) {
                         // 8-byte reads from unrelated base registers (one per contraction step and
                         // half): fused in pairs into ds_read2_b64 they would conflict on the LDS
                         // banks at this row stride
                         const unsigned lo = opaque(xq + 32 * ks * E), hi = opaque(xq + (32 * ks + 16) * E);
-                        bx[ks][i4] = cat<V8, V4>(ld4(lo + 16 * i4 * XS * E), ld4(hi + 16 * i4 * XS * E));
+                        bx[ks % NBX][i4] = cat<V8, V4>(ld4(lo + 16 * i4 * XS * E), ld4(hi + 16 * i4 * XS * E));
                     }
                     __builtin_amdgcn_sched_barrier(0);  // (keeps the address registers of one step at a time)
-                }
-                __builtin_amdgcn_sched_barrier(0);
-                f32x4 oacc[4];
+                };
+                auto read_p = [&]() {
 #pragma unroll
-                for (int i4 = 0; i4 < 4; ++i4) oacc[i4] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                    for (int i4 = 0; i4 < 4; ++i4) {
+#pragma unroll
+                        for (int k2 = 0; k2 < 2; ++k2) {
+                            const bool need = REVERSE ? (k2 >= i4 / 2) : (k2 <= i4 / 2);
+                            if (need) bp[i4][k2] = ld8(pq + (16 * i4 * PS + 32 * k2) * E);
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                };
+#pragma unroll
+                for (int ks = 0; ks < (NH == 1 ? KS : 1); ++ks) read_x(ks);
+                f32x4 oacc[NH][4];
+#pragma unroll
+                for (int h = 0; h < NH; ++h)
+#pragma unroll
+                    for (int i4 = 0; i4 < 4; ++i4) oacc[h][i4] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    V8 sb;
+                    if (NH > 1 && ks + 1 < KS) read_x(ks + 1);
+                    V8 sb[NH];
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        sb[v] = M::cvt(st[2 * ks][v]);
-                        sb[4 + v] = M::cvt(st[2 * ks + 1][v]);
-                    }
+                    for (int h = 0; h < NH; ++h)
 #pragma unroll
-                    for (int i4 = 0; i4 < 4; ++i4) oacc[i4] = M::mma(sb, bx[ks][i4], oacc[i4]);
-                    if (ks == (KS - 1) / 2) {
-                        // the P fragments follow once half of the x fragments have been used up
-                        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                        for (int i4 = 0; i4 < 4; ++i4) {
-#pragma unroll
-                            for (int k2 = 0; k2 < 2; ++k2) {
-                                const bool need = REVERSE ? (k2 >= i4 / 2) : (k2 <= i4 / 2);
-                                if (need) bp[i4][k2] = ld8(pq + (16 * i4 * PS + 32 * k2) * E);
-                            }
+                        for (int v = 0; v < 4; ++v) {
+                            sb[h][v] = M::cvt(st[h][2 * ks][v]);
+                            sb[h][4 + v] = M::cvt(st[h][2 * ks + 1][v]);
                         }
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-                if (DECAY) {
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int i4 = 0; i4 < 4; ++i4)
 #pragma unroll
-                        for (int v = 0; v < 4; ++v) oacc[i4][v] *= cf[i4];
+                        for (int h = 0; h < NH; ++h) oacc[h][i4] = M::mma(sb[h], bx[ks % NBX][i4], oacc[h][i4]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    // the P fragments follow once half of the x fragments have been used up
+                    if (NH == 1 && ks == (KS - 1) / 2) read_p();
+                }
+                if (NH > 1) read_p();
+                if (DECAY) {
+#pragma unroll
+                    for (int h = 0; h < NH; ++h)
+#pragma unroll
+                        for (int i4 = 0; i4 < 4; ++i4)
+#pragma unroll
+                            for (int v = 0; v < 4; ++v) oacc[h][i4][v] *= cf[i4];
                 }
 #pragma unroll
                 for (int i4 = 0; i4 < 4; ++i4) {
 #pragma unroll
                     for (int ks = 0; ks < 2; ++ks) {
                         const bool need = REVERSE ? (ks >= i4 / 2) : (ks <= i4 / 2);
-                        if (need) oacc[i4] = M::mma(zf[ks], bp[i4][ks], oacc[i4]);
+#pragma unroll
+                        for (int h = 0; h < NH; ++h)
+                            if (need) oacc[h][i4] = M::mma(zf[h][ks], bp[i4][ks], oacc[h][i4]);
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 // leave the tile in the z slot of this block, over this wave's own z columns (read
                 // above, and by no other wave); the next iteration's staging sends it to memory
-                const unsigned oq = opaque(ZBASE + bcur * ZTB + lane_ow);
+                const unsigned oq = opaque(ZBASE + zcur * ZTB + lane_ow);
 #pragma unroll
-                for (int i4 = 0; i4 < 4; ++i4) {
-                    V4 o;
+                for (int h = 0; h < NH; ++h)
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) o[v] = (T)oacc[i4][v];
-                    *reinterpret_cast<V4*>(smem + oq + 16 * i4 * ZS * E) = o;
-                }
+                    for (int i4 = 0; i4 < 4; ++i4) {
+                        V4 o;
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) o[v] = (T)oacc[h][i4][v];
+                        *reinterpret_cast<V4*>(smem + oq + (16 * i4 * ZS + 16 * h) * E) = o;
+                    }
             }
             if (have_next) {
                 // state = lam^64 state + y^T (z * Lupd)
@@ -467,18 +487,23 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
                 __builtin_amdgcn_sched_barrier(0);
                 if (DECAY) {
 #pragma unroll
-                    for (int ks = 0; ks < 2; ++ks)
+                    for (int h = 0; h < NH; ++h) {
 #pragma unroll
-                        for (int u = 0; u < 8; ++u) zf[ks][u] = (T)((float)zf[ks][u] * cf[4 + 8 * ks + u]);
+                        for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-                    for (int kt = 0; kt < KT; ++kt)
+                            for (int u = 0; u < 8; ++u) zf[h][ks][u] = (T)((float)zf[h][ks][u] * cf[4 + 8 * ks + u]);
 #pragma unroll
-                        for (int v = 0; v < 4; ++v) st[kt][v] *= lamB;
+                        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                            for (int v = 0; v < 4; ++v) st[h][kt][v] *= lamB;
+                    }
                 }
 #pragma unroll
                 for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
-                    for (int ks = 0; ks < 2; ++ks) st[kt] = M::mma(ay[kt][ks], zf[ks], st[kt]);
+                    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                        for (int h = 0; h < NH; ++h) st[h][kt] = M::mma(ay[kt][ks], zf[h][ks], st[h][kt]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -500,29 +525,48 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
     // the last block's output tile is still in its z slot when the walk ends
     auto flush_last = [&]() {
         if (it_end <= it_first) return;
-        const unsigned zd = ZBASE + (unsigned)((it_end - 1) % 3) * ZTB + lane_stage_z;
+        const unsigned zd = ZBASE + (unsigned)(NH == 1 ? (it_end - 1) % 3 : (it_end - 1) & 1) * ZTB + lane_stage_z;
         u32x4 o[ZC];
 #pragma unroll
-        for (int u = 0; u < ZC; ++u) o[u] = *reinterpret_cast<const u32x4*>(smem + zd + u * (NL / 8) * ZS * E);
+        for (int u = 0; u < ZC; ++u) o[u] = *reinterpret_cast<const u32x4*>(smem + zd + u * ZROWS * ZS * E);
         store_out(it_end - 1, true, o);
     };
-    if (state_role) {
+    // The two kinds of waves part here for good, prologue included (two barriers in each branch):
+    // the compiler lays the branches out one after the other and keeps alive, while the first one
+    // runs, whatever the second one needs of the values computed before this point - which must
+    // therefore not include the score waves' prefetch registers.
+    if (!state_role) {
+        load_block(0, xrA, yrA, zrA);
+        load_block(1, xrB, yrB, zrB);
+        stage_block(0, NH == 1 ? 0 : 1, xrA, yrA, zrA, 0, false);
+        load_block(2, xrA, yrA, zrA);
+        stage_block(1, NH == 1 ? 1 : 0, xrB, yrB, zrB, 0, false);
+        load_block(3, xrB, yrB, zrB);
+        __syncthreads();
+        if (it_first == 0) score_block(0, 0);
+        __syncthreads();
+        walk(std::false_type{});
+        flush_last();
+    } else {
+        __syncthreads();
+        __syncthreads();
         // The state waves are the critical path and every SIMD holds one wave of each kind: when both
         // have an instruction ready (right after the barrier all eight waves go for LDS), theirs goes first.
         __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+        for (int h = 0; h < NH; ++h)
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) st[h][kt] = (f32x4){0.f, 0.f, 0.f, 0.f};
         walk(std::true_type{});
-    } else {
-        walk(std::false_type{});
-        flush_last();
     }
 }
 
-template <typename T, int DKP, bool REVERSE, bool DECAY, bool DENSE>
+template <typename T, int DKP, int NH, bool REVERSE, bool DECAY, bool DENSE>
 static int launch_one(const SweepPair& pair, hipStream_t st) {
     const SweepArgs& a = pair.a[0];
-    constexpr size_t lds = PipeLds<DKP>::bytes(sizeof(T));
+    constexpr size_t lds = PipeLds<DKP, NH>::bytes(sizeof(T));
     static_assert(lds <= 160 * 1024, "LDS budget");
-    auto kern = la_sweep_pipe_kernel<T, DKP, REVERSE, DECAY, DENSE>;
+    auto kern = la_sweep_pipe_kernel<T, DKP, NH, REVERSE, DECAY, DENSE>;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -548,10 +592,11 @@ static int launch_dir(const SweepPair& pair, hipStream_t st) {
         dense = dense && plain(c.lx, c.h, c.n, c.dk) && plain(c.ly, c.h, c.n, c.dk) && plain(c.lz, c.h, c.n, c.dv) &&
                 plain(c.lo, c.h, c.n, c.dv);
     }
-#define LA_GO2(DKP, DENSE) (decay ? launch_one<T, DKP, REVERSE, true, DENSE>(pair, st) : launch_one<T, DKP, REVERSE, false, DENSE>(pair, st))
-#define LA_GO(DKP) (dense ? LA_GO2(DKP, true) : LA_GO2(DKP, false))
-    if (a.dk <= 64) return LA_GO(64);
-    return LA_GO(128);
+#define LA_GO2(DKP, NH, DENSE) (decay ? launch_one<T, DKP, NH, REVERSE, true, DENSE>(pair, st) : launch_one<T, DKP, NH, REVERSE, false, DENSE>(pair, st))
+#define LA_GO(DKP, NH) (dense ? LA_GO2(DKP, NH, true) : LA_GO2(DKP, NH, false))
+    if (pair.wide) return LA_GO(128, 2);  // 128 columns per workgroup (nslice counts those)
+    if (a.dk <= 64) return LA_GO(64, 1);
+    return LA_GO(128, 1);
 #undef LA_GO
 #undef LA_GO2
 }

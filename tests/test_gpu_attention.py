@@ -268,19 +268,48 @@ def test_chunked_walk_on_projection_layout(chunks, monkeypatch):
     check(got, want, torch.bfloat16, "chunked token-major")
 
 
-@pytest.mark.parametrize("b, h, n, d", [(2, 4, 1000, 128), (1, 3, 777, 64), (1, 2, 500, 192), (1, 2, 300, 256)])
+@pytest.mark.parametrize("b, h, n, d", [(2, 4, 1000, 128), (1, 3, 777, 64), (1, 2, 500, 192), (1, 2, 300, 256),
+                                        (1, 5, 913, 72), (2, 3, 450, 96), (1, 2, 1100, 120)])
 def test_paired_backward_launch_matches_separate_launches(b, h, n, d, monkeypatch):
     """With d == e the dK and dV sweeps travel in one launch (their workgroups share the reads of dO
-    and q); LA_SWEEP_UNPAIRED=1 launches them one after the other.  Same numbers, bit for bit."""
+    and q), with 64 or - LA_SWEEP_WIDE=1 - 128 columns per workgroup; LA_SWEEP_UNPAIRED=1 launches
+    them one after the other.  Same numbers, bit for bit, also when the walk is cut into chunks."""
     q, k, v, do = make_inputs(b, h, n, d, d, torch.bfloat16, 1.0, seed=d + n)
     s = _build_slope_tensor(h)
-    monkeypatch.delenv("LA_SWEEP_UNPAIRED", raising=False)
-    paired = run_hip(q, k, v, s, do)
-    monkeypatch.setenv("LA_SWEEP_UNPAIRED", "1")
-    separate = run_hip(q, k, v, s, do)
-    monkeypatch.delenv("LA_SWEEP_UNPAIRED", raising=False)
-    for a, c in zip(paired, separate):
+    got = {}
+    for mode, env in (("narrow", {"LA_SWEEP_WIDE": "0"}), ("wide", {"LA_SWEEP_WIDE": "1"}),
+                      ("wide chunked", {"LA_SWEEP_WIDE": "1", "LA_SWEEP_CHUNKS": "3"}), ("separate", {"LA_SWEEP_UNPAIRED": "1"})):
+        for name in ("LA_SWEEP_WIDE", "LA_SWEEP_CHUNKS", "LA_SWEEP_UNPAIRED"):
+            monkeypatch.delenv(name, raising=False)
+        for name, value in env.items():
+            monkeypatch.setenv(name, value)
+        got[mode] = run_hip(q, k, v, s, do)
+    for name in ("LA_SWEEP_WIDE", "LA_SWEEP_CHUNKS", "LA_SWEEP_UNPAIRED"):
+        monkeypatch.delenv(name, raising=False)
+    for mode in ("narrow", "wide", "wide chunked"):
+        for a, c in zip(got[mode], got["separate"]):
+            assert torch.equal(a, c), mode
+    if d <= 128:
+        want = oracle.linear_attn_fwd_bwd(q, k, v, s, do, torch.float32)
+        check(got["wide"], want, torch.bfloat16, "wide pair d=%d" % d)
+
+
+def test_wide_pair_on_token_major_tensors(monkeypatch):
+    """The 128-column workgroups on strided tensors (explicit row masks, ragged n)."""
+    b, h, n, d = 1, 3, 1237, 128
+    g = torch.Generator().manual_seed(29)
+    q, k = ((torch.randn(b, n, h, d, generator=g) * 0.7).bfloat16().to(DEV).transpose(1, 2) for _ in range(2))
+    v, do = (torch.randn(b, n, h, d, generator=g).bfloat16().to(DEV).transpose(1, 2) for _ in range(2))
+    s = _build_slope_tensor(h)
+    monkeypatch.setenv("LA_SWEEP_WIDE", "1")
+    wide = run_hip(q.detach(), k.detach(), v.detach(), s, do)
+    monkeypatch.setenv("LA_SWEEP_WIDE", "0")
+    narrow = run_hip(q.detach(), k.detach(), v.detach(), s, do)
+    monkeypatch.delenv("LA_SWEEP_WIDE", raising=False)
+    for a, c in zip(wide, narrow):
         assert torch.equal(a, c)
+    want = oracle.linear_attn_fwd_bwd(q.cpu(), k.cpu(), v.cpu(), s, do.cpu(), torch.float32)
+    check(wide, want, torch.bfloat16, "wide token-major")
 
 
 def test_deterministic():
