@@ -2,24 +2,27 @@
 // software-pipelined variant with one workgroup barrier per 64-token block.
 //
 // Same operator and the same division of the data as la_sweep.hip (one workgroup of
-// 8 wavefronts per (batch, head, 64-column slice of z/out), 64-token blocks walked in
-// order, fp32 state in MFMA accumulators), but the two kinds of wavefronts work on
+// 8 wavefronts per (batch, head, 64- or 128-column slice of z/out), 64-token blocks walked
+// in order, fp32 state in MFMA accumulators), but the two kinds of wavefronts work on
 // different blocks at the same time:
 //   waves 0-3 ("score" waves)  do all the memory traffic (fetch blocks it+3 / it+4 into two
 //                              register sets, publish block it+2 in LDS, write the output
 //                              tile of block it-1 back) and, during iteration `it`, compute
 //                              the masked, decayed score tile P of block it+1 into LDS;
-//   waves 4-7 ("state" waves)  own a dk x 16 column slab of the state and finish block
-//                              `it`: out^T = Lout * (state^T x^T) + z^T P^T, left in LDS,
-//                              then state = lam^64 state + y^T (z * Lupd).
+//   waves 4-7 ("state" waves)  own one or two dk x 16 column slabs of the state and finish
+//                              block `it`: out^T = Lout * (state^T x^T) + z^T P^T, left in
+//                              LDS, then state = lam^64 state + y^T (z * Lupd).
 // The inter-block term therefore never leaves registers, the state waves' serial chain holds
 // no memory instructions, and a single barrier per iteration orders
 //   - the x/y/z tiles: three LDS buffers (block `it` read by the state waves, block it+1
 //     read by the score waves, block it+2 being written);
 //   - the P tiles: two LDS buffers (block `it` read, block it+1 written);
 //   - the output tile of block `it`, which the state waves write over the z columns they
-//     alone read and which leaves for memory as whole 128-byte row segments when that z slot
-//     is refilled one iteration later.
+//     alone read and which leaves for memory as whole row segments when that z slot is
+//     refilled one iteration later.
+// The chip runs this kernel at its socket power limit, so what counts is the work per output
+// element (LDS traffic above all), not the length of any dependency chain: hence the 128-column
+// form wherever the launch still has a workgroup for every CU.
 // (lightning_attn/ops/triton/lightning_attn2.py:8-85 forward, :88-395 backward.)
 #include <type_traits>
 
