@@ -1,0 +1,65 @@
+"""The C entry points only enqueue kernels on the stream they are given: no allocation, no
+synchronisation, no memset.  A forward + backward pair therefore records into a HIP graph, and every
+replay must reproduce the eager result for the data then in the buffers."""
+import os
+import sys
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "lightning-attention_amd"))
+
+from lightning_attn.ops import lightning_attn_func  # noqa: E402
+from lightning_attn.ops.hip import _lib  # noqa: E402
+from lightning_attn.utils import _build_slope_tensor  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("b, h, n, d", [(2, 4, 700, 128), (1, 6, 1000, 64), (1, 2, 400, 192)])
+def test_forward_backward_replay_from_a_graph(b, h, n, d):
+    dev = torch.device("cuda")
+    L = _lib.lib()
+    code = _lib.dtype_code(torch.bfloat16)
+    g = torch.Generator(device=dev).manual_seed(5)
+
+    def fresh():
+        return tuple((torch.randn(b, h, n, d, generator=g, device=dev) * sc).bfloat16() for sc in (0.6, 0.6, 1.0, 1.0))
+
+    q, k, v, do = fresh()
+    o, dq, dk, dv = (torch.empty_like(q) for _ in range(4))
+    s = _build_slope_tensor(h).to(dev).reshape(h).contiguous()
+
+    def enqueue():
+        st = _lib.stream_ptr(dev)
+        _lib.check(L.la_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr(), o.data_ptr(), b, h, n, d, d, code,
+                            None, 0, st), "la_fwd")
+        _lib.check(L.la_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr(), do.data_ptr(), dq.data_ptr(),
+                            dk.data_ptr(), dv.data_ptr(), b, h, n, d, d, code, None, 0, st), "la_bwd")
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        enqueue()  # first use outside the capture: function attributes, device queries
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        enqueue()
+
+    for rep in range(3):
+        for dst, src in zip((q, k, v, do), fresh()):
+            dst.copy_(src)
+        for t in (o, dq, dk, dv):
+            t.fill_(float("nan"))  # a fill kernel, not a memset node
+        graph.replay()
+        torch.cuda.synchronize()
+        # the same numbers through the eager operator
+        qe, ke, ve = (t.clone().requires_grad_() for t in (q, k, v))
+        oe = lightning_attn_func(qe, ke, ve, s)
+        oe.backward(do)
+        torch.cuda.synchronize()
+        for name, a, c in zip(("o", "dq", "dk", "dv"), (o, dq, dk, dv), (oe.detach(), qe.grad, ke.grad, ve.grad)):
+            assert torch.equal(a, c), (rep, name)
