@@ -212,25 +212,6 @@ def main():
         out["fwd_ms"] = round(event_ms(lambda: lightning_attn_func(q, k, v, s), 20), 4)
         out["bwd_ms"] = round(event_ms(bwd_only, 20), 4)
         del o
-        # the same three launches (la_fwd + la_bwd through the C ABI) recorded once into a HIP graph and
-        # replayed: the step without the host side of autograd and without launch gaps (for reference only)
-        gq, gk, gv, gdo = (t.detach() for t in (q, k, v, do))
-        go, gdq, gdk, gdv = (torch.empty_like(gq) for _ in range(4))
-
-        def enqueue():
-            sp = torch.cuda.current_stream().cuda_stream
-            assert L.la_fwd(gq.data_ptr(), gk.data_ptr(), gv.data_ptr(), s.data_ptr(), go.data_ptr(), B, H, N, D, D, 0,
-                            None, 0, sp) == 0
-            assert L.la_bwd(gq.data_ptr(), gk.data_ptr(), gv.data_ptr(), s.data_ptr(), gdo.data_ptr(), gdq.data_ptr(),
-                            gdk.data_ptr(), gdv.data_ptr(), B, H, N, D, D, 0, None, 0, sp) == 0
-
-        enqueue()
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            enqueue()
-        out["graph_replay_step_ms"] = round(event_ms(graph.replay, 30), 4)
-        del graph, go, gdq, gdk, gdv
         sweep = {}
         for n in (512, 1024, 2048, 4096, 8192, 16384, 32768):
             q = k = v = do = None
