@@ -294,13 +294,14 @@ def test_paired_backward_launch_matches_separate_launches(b, h, n, d, monkeypatc
         check(got["wide"], want, torch.bfloat16, "wide pair d=%d" % d)
 
 
-def test_many_sequences_take_the_128_column_workgroups():
+@pytest.mark.parametrize("dtype, decay", [(torch.bfloat16, True), (torch.float16, True), (torch.bfloat16, False)])
+def test_many_sequences_take_the_128_column_workgroups(dtype, decay):
     """b * h >= the number of CUs: the library picks 128-column workgroups for every launch by itself."""
     b, h, n, d = 32, 8, 130, 128
-    q, k, v, do = make_inputs(b, h, n, d, d, torch.bfloat16, 1.0, seed=77)
-    s = _build_slope_tensor(h)
+    q, k, v, do = make_inputs(b, h, n, d, d, dtype, 1.0 if dtype == torch.bfloat16 else 0.5, seed=77)
+    s = _build_slope_tensor(h) if decay else None
     want = oracle.linear_attn_fwd_bwd(q, k, v, s, do, torch.float32)
-    check(run_hip(q, k, v, s, do), want, torch.bfloat16, "many sequences")
+    check(run_hip(q, k, v, s, do), want, dtype, "many sequences")
 
 
 def test_wide_pair_on_token_major_tensors(monkeypatch):
