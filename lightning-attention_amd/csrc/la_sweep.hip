@@ -490,11 +490,6 @@ static int launch_dir(const SweepPair& pair, hipStream_t st) {
 #undef LA_GO
 }
 
-// Sequence chunks per (batch, head, slice).  With few sequences a single sweep per sequence
-// leaves most of the 256 CUs idle; the walk is then cut into up to 8 chunks whose workgroups
-// rebuild their incoming state themselves.  A warm-up block costs about half a full block, so
-// chunk lengths shrink geometrically (len_c ~ (1 - rho)^c, rho = 0.5) to make all workgroups
-// finish together.  LA_SWEEP_CHUNKS=<C> overrides the count.
 static int num_cus() {
     static const int cus = [] {
         int dev = 0, n = 256;
@@ -504,6 +499,11 @@ static int num_cus() {
     return cus;
 }
 
+// Sequence chunks per (batch, head, slice).  With few sequences a single sweep per sequence
+// leaves most of the 256 CUs idle; the walk is then cut into up to 8 chunks whose workgroups
+// rebuild their incoming state themselves.  A warm-up block costs about half a full block, so
+// chunk lengths shrink geometrically (len_c ~ (1 - rho)^c, rho = 0.5) to make all workgroups
+// finish together.  LA_SWEEP_CHUNKS=<C> overrides the count.
 static void choose_chunks(SweepArgs& a, int nprod = 1) {
     const char* env = getenv("LA_SWEEP_CHUNKS");  // read per call so that tests can vary it
     const int forced = env ? atoi(env) : 0;
@@ -539,15 +539,19 @@ static void choose_chunks(SweepArgs& a, int nprod = 1) {
     for (int i = (int)c + 1; i < 9; ++i) a.chunk_start[i] = (int)nblk;
 }
 
-// Where 128-column workgroups still fill the chip, the pipelined kernel gives each workgroup 128
-// columns of z / out instead of 64: the score tile and the x / y tiles are then produced once per
-// 128 output columns, and the power-limited kernel turns the saved work into time (dK + dV at the
-// headline shape: 0.31 against 0.415 ms).  LA_SWEEP_WIDE=0 / 1 overrides the choice.
+// The pipelined kernel can give each workgroup 128 columns of z / out instead of 64: the score tile
+// and the x / y tiles are then produced once per 128 output columns, and the power-limited kernel
+// turns the saved work into time (dK + dV at the headline shape: 0.31 against 0.415 ms) - as long
+// as there are workgroups enough.  A 128-column workgroup takes about 1.25 times as long as a
+// 64-column one, and there are half as many: compare the rounds of workgroups the chip has to run.
+// LA_SWEEP_WIDE=0 / 1 overrides the choice.
 static bool wide_columns(int64_t bh, int64_t dk, int64_t dv, int nprod) {
     if (dk > 128 || dv <= 64 || dv > 128) return false;
     const char* env = getenv("LA_SWEEP_WIDE");
     if (env) return atoi(env) != 0;
-    return (int64_t)((bh + 7) / 8 * 8) * nprod >= num_cus();
+    const int64_t cus = num_cus(), wide = (bh + 7) / 8 * 8 * nprod, narrow = 2 * wide;
+    if (narrow <= cus) return false;  // every 64-column workgroup gets a CU of its own
+    return (wide + cus - 1) / cus * 5 < (narrow + cus - 1) / cus * 4;
 }
 
 static SweepArgs make_args(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv) {
