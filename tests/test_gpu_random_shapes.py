@@ -1,0 +1,68 @@
+"""Seeded random walk over shapes, dtypes, layouts and launch modes (sequence chunks, 64- / 128-column
+workgroups, paired / separate dK + dV launches), each case against the naive oracle."""
+import os
+import random
+import sys
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "lightning-attention_amd"))
+sys.path.insert(0, ROOT)
+
+from lightning_attn.ops import lightning_attn_func  # noqa: E402
+from lightning_attn.utils import _build_slope_tensor  # noqa: E402
+from oracle import linear_attn_oracle as oracle  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+KNOBS = ("LA_SWEEP_WIDE", "LA_SWEEP_CHUNKS", "LA_SWEEP_UNPAIRED")
+
+
+def _rel(a, r):
+    return ((a.float().cpu() - r.float()).norm() / (r.float().norm() + 1e-30)).item()
+
+
+@pytest.mark.parametrize("seed", [101, 202, 303])
+def test_random_cases_match_the_oracle(seed, monkeypatch):
+    rnd = random.Random(seed)
+    for case in range(14):
+        b, h = rnd.randint(1, 3), rnd.randint(1, 9)
+        n = rnd.choice([1, 2, 63, 64, 65, 127, 128, 129, 300, 513, 777, 1000, rnd.randint(1, 1200)])
+        d = 8 * rnd.randint(1, 32)
+        e = d if rnd.random() < 0.6 else 8 * rnd.randint(1, 32)
+        dtype = rnd.choice([torch.bfloat16, torch.bfloat16, torch.float16])
+        decay = rnd.random() < 0.75
+        token_major = rnd.random() < 0.4
+        env = {}
+        if rnd.random() < 0.6:
+            env["LA_SWEEP_WIDE"] = rnd.choice(["0", "1"])
+        if rnd.random() < 0.5:
+            env["LA_SWEEP_CHUNKS"] = str(rnd.randint(1, 5))
+        if rnd.random() < 0.2:
+            env["LA_SWEEP_UNPAIRED"] = "1"
+        for name in KNOBS:
+            monkeypatch.delenv(name, raising=False)
+        for name, value in env.items():
+            monkeypatch.setenv(name, value)
+        g = torch.Generator().manual_seed(1000 * seed + case)
+
+        def make(cols, scale):
+            t = (torch.randn(b, n, h, cols, generator=g) * scale).to(dtype)
+            return t.to(DEV).transpose(1, 2) if token_major else t.transpose(1, 2).contiguous().to(DEV)
+
+        q, k, v, do = make(d, 0.6), make(d, 0.6), make(e, 1.0), make(e, 1.0)
+        s = _build_slope_tensor(h) if decay else None
+        what = (seed, case, (b, h, n, d, e), dtype, decay, token_major, env)
+        print(what, flush=True)  # names the case should a launch go wrong
+        qg, kg, vg = (t.detach().requires_grad_() for t in (q, k, v))
+        o = lightning_attn_func(qg, kg, vg, None if s is None else s.to(DEV))
+        o.backward(do)
+        torch.cuda.synchronize()
+        want = oracle.linear_attn_fwd_bwd(q.cpu(), k.cpu(), v.cpu(), s, do.cpu(), torch.float32)
+        limit = 1e-2 if dtype == torch.bfloat16 else 2e-3
+        for name, a, r in zip(("o", "dq", "dk", "dv"), (o.detach(), qg.grad, kg.grad, vg.grad), want):
+            assert a.dtype == dtype and _rel(a, r) < limit, (what, name, _rel(a, r))
+    for name in KNOBS:
+        monkeypatch.delenv(name, raising=False)
