@@ -244,8 +244,8 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
     // Publishes a fetched block in tile buffer `buf`.  The z slot of that buffer still holds the
     // output tile of the block that used it last (walk index bout; the state waves leave their
     // columns of `out` there, over the z columns they alone read): every thread first takes the 16
-    // bytes its z chunk is about to replace and, if `flush`, sends them to memory - eight lanes
-    // write one whole 128-byte row segment.  (Stored straight from the accumulators, each wave
+    // bytes its z chunk is about to replace and, if `flush`, sends them to memory - eight (NH = 2:
+    // sixteen) lanes write one whole 128-byte (256-byte) row segment.  (Stored straight from the accumulators, each wave
     // would write 32-byte pieces of every row, which the memory system handles far worse: 0.083
     // against 0.048 ms for the output traffic alone at the headline shape.)
     const unsigned lane_o = lane_zcol < dv ? (lane_zrow * ots + lane_zcol) * (unsigned)sizeof(T) : kOob;
