@@ -2,7 +2,10 @@
 //
 // One 64-lane wavefront owns one row: the row is read once with 16-byte loads
 // straight into registers, reduced with cross-lane shuffles (no LDS, no
-// barrier), and written once.  Four rows per 256-thread workgroup.
+// barrier), and written once.  Two rows per 128-thread workgroup.  Only the packed
+// inputs are kept across the reduction (the second pass converts them again):
+// carrying the converted floats cost the backward kernel 168 registers and half
+// of its waves in flight (5.7 -> 6.2 TB/s with 79 registers).
 // Replaces srms_norm_fw / srms_norm_bwd_dx_fused
 // (lightning_attn/ops/triton/srmsnorm.py:12-33, 38-74).
 #include "la_common.h"
@@ -30,13 +33,22 @@ __device__ __forceinline__ void store16(T* p, const Pack16<T>& r) {
 }
 
 // ---- register-resident rows: cols <= 64 * (16/sizeof T) * NV ---------------
+constexpr int kRowsPerGroup = 2;
+
+// Makes the optimiser forget what it knows about a packed register quartet, so that values derived
+// from it before this point (float conversions) are not kept alive for later use.
+template <typename T>
+__device__ __forceinline__ void forget(Pack16<T>& p) {
+    asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&p)));
+}
+
 template <typename T, int NV>
-__global__ __launch_bounds__(256) void srms_fwd_vec(const T* __restrict__ x, T* __restrict__ y,
+__global__ __launch_bounds__(64 * kRowsPerGroup) void srms_fwd_vec(const T* __restrict__ x, T* __restrict__ y,
                                                     float* __restrict__ rstd, int64_t rows, int cols,
                                                     int64_t stride, float eps) {
     constexpr int E = Pack16<T>::N;
     const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t row = (int64_t)blockIdx.x * kRowsPerGroup + (threadIdx.x >> 6);
     if (row >= rows) return;
     const T* xr = x + row * stride;
     T* yr = y + row * stride;
@@ -62,6 +74,8 @@ __global__ __launch_bounds__(256) void srms_fwd_vec(const T* __restrict__ x, T* 
     const float rs = 1.0f / sqrtf(ss / (float)cols + eps);
     if (lane == 0) rstd[row] = rs;
 #pragma unroll
+    for (int u = 0; u < NV; ++u) forget(buf[u]);
+#pragma unroll
     for (int u = 0; u < NV; ++u) {
         const int c = (u * 64 + lane) * E;
         if (c < cols) {
@@ -74,12 +88,12 @@ __global__ __launch_bounds__(256) void srms_fwd_vec(const T* __restrict__ x, T* 
 }
 
 template <typename T, int NV>
-__global__ __launch_bounds__(256) void srms_bwd_vec(const T* __restrict__ x, const T* __restrict__ dy,
+__global__ __launch_bounds__(64 * kRowsPerGroup) void srms_bwd_vec(const T* __restrict__ x, const T* __restrict__ dy,
                                                     const float* __restrict__ rstd, T* __restrict__ dx,
                                                     int64_t rows, int cols, int64_t stride) {
     constexpr int E = Pack16<T>::N;
     const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t row = (int64_t)blockIdx.x * kRowsPerGroup + (threadIdx.x >> 6);
     if (row >= rows) return;
     const T* xr = x + row * stride;
     const T* gr = dy + row * (int64_t)cols;  // dy and dx are dense (rows, cols)
@@ -105,6 +119,11 @@ __global__ __launch_bounds__(256) void srms_bwd_vec(const T* __restrict__ x, con
     }
     acc = wave_sum(acc);
     const float m = acc / (float)cols;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        forget(bx[u]);
+        forget(bg[u]);
+    }
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
         const int c = (u * 64 + lane) * E;
@@ -179,9 +198,9 @@ static int launch_fwd(const void* x, void* y, float* rstd, int64_t rows, int64_t
     T* yp = static_cast<T*>(y);
     const bool vec = (cols % E == 0) && (stride % E == 0) && aligned16(x) && aligned16(y) && cols <= 64 * E * 16;
     if (vec) {
-        const unsigned grid = (unsigned)((rows + 3) / 4);
+        const unsigned grid = (unsigned)((rows + kRowsPerGroup - 1) / kRowsPerGroup);
         const int nv = (int)((cols + 64 * E - 1) / (64 * E));
-#define LA_FWD(NV) hipLaunchKernelGGL((srms_fwd_vec<T, NV>), dim3(grid), dim3(256), 0, st, xp, yp, rstd, rows, (int)cols, stride, eps)
+#define LA_FWD(NV) hipLaunchKernelGGL((srms_fwd_vec<T, NV>), dim3(grid), dim3(64 * kRowsPerGroup), 0, st, xp, yp, rstd, rows, (int)cols, stride, eps)
         if (nv <= 1) LA_FWD(1);
         else if (nv <= 2) LA_FWD(2);
         else if (nv <= 4) LA_FWD(4);
@@ -204,9 +223,9 @@ static int launch_bwd(const void* x, const void* dy, const float* rstd, void* dx
     const bool vec = (cols % E == 0) && (stride % E == 0) && aligned16(x) && aligned16(dy) && aligned16(dx) &&
                      cols <= 64 * E * 8;
     if (vec) {
-        const unsigned grid = (unsigned)((rows + 3) / 4);
+        const unsigned grid = (unsigned)((rows + kRowsPerGroup - 1) / kRowsPerGroup);
         const int nv = (int)((cols + 64 * E - 1) / (64 * E));
-#define LA_BWD(NV) hipLaunchKernelGGL((srms_bwd_vec<T, NV>), dim3(grid), dim3(256), 0, st, xp, gp, rstd, dp, rows, (int)cols, stride)
+#define LA_BWD(NV) hipLaunchKernelGGL((srms_bwd_vec<T, NV>), dim3(grid), dim3(64 * kRowsPerGroup), 0, st, xp, gp, rstd, dp, rows, (int)cols, stride)
         if (nv <= 1) LA_BWD(1);
         else if (nv <= 2) LA_BWD(2);
         else if (nv <= 4) LA_BWD(4);
