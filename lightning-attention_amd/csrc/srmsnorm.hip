@@ -1,11 +1,13 @@
 // SimpleRMSNorm forward / backward row kernels for gfx950.
 //
-// One 64-lane wavefront owns one row: the row is read once with 16-byte loads
-// straight into registers, reduced with cross-lane shuffles (no LDS, no
-// barrier), and written once.  Two rows per 128-thread workgroup.  Only the packed
-// inputs are kept across the reduction (the second pass converts them again):
-// carrying the converted floats cost the backward kernel 168 registers and half
-// of its waves in flight (5.7 -> 6.2 TB/s with 79 registers).
+// A row is read once with 16-byte loads straight into registers, reduced, and
+// written once.  Up to 1024 chunks of 16 bytes: one 64-lane wavefront per row and
+// workgroup, cross-lane shuffles, no LDS, no barrier (one row per workgroup measured
+// against 2, 4 and 8 at 1024 to 4096 columns: never slower); short rows share a
+// wavefront (4 .. 32 lanes each); rows up to 64 KB take a four-wavefront workgroup.
+// Only the packed inputs are kept across the reduction (the second pass converts them
+// again): carrying the converted floats cost the backward kernel 168 registers and
+// half of its waves in flight (5.7 -> 6.2 TB/s with 79 registers).
 // Replaces srms_norm_fw / srms_norm_bwd_dx_fused
 // (lightning_attn/ops/triton/srmsnorm.py:12-33, 38-74).
 #include "la_common.h"
@@ -32,8 +34,10 @@ __device__ __forceinline__ void store16(T* p, const Pack16<T>& r) {
     __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(&r), reinterpret_cast<u32x4*>(p));
 }
 
-// ---- register-resident rows: cols <= 64 * (16/sizeof T) * NV ---------------
-constexpr int kRowsPerGroup = 2;
+// ---- register-resident rows -------------------------------------------------
+// TPR threads share a row (4 .. 64: 64 / TPR rows per single-wavefront workgroup, cross-lane
+// reduction; 256: one four-wavefront workgroup per row, reduction through LDS), each holding NV
+// 16-byte chunks of it: cols <= TPR * NV * (16 / sizeof T).
 
 // Makes the optimiser forget what it knows about a packed register quartet, so that values derived
 // from it before this point (float conversions) are not kept alive for later use.
@@ -42,27 +46,47 @@ __device__ __forceinline__ void forget(Pack16<T>& p) {
     asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&p)));
 }
 
-template <typename T, int NV>
-__global__ __launch_bounds__(64 * kRowsPerGroup) void srms_fwd_vec(const T* __restrict__ x, T* __restrict__ y,
-                                                    float* __restrict__ rstd, int64_t rows, int cols,
-                                                    int64_t stride, float eps) {
+__device__ __forceinline__ float block_sum_256(float v, float* red) {
+    v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    const float t = red[0] + red[1] + red[2] + red[3];
+    __syncthreads();
+    return t;
+}
+
+// sum over the TPR threads of a row (every thread of the workgroup takes part)
+template <int TPR>
+__device__ __forceinline__ float row_sum(float v, float* red) {
+    if (TPR == 256) return block_sum_256(v, red);
+#pragma unroll
+    for (int m = TPR / 2; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+    return v;
+}
+
+template <typename T, int NV, int TPR>
+__global__ __launch_bounds__(TPR == 256 ? 256 : 64) void srms_fwd_vec(const T* __restrict__ x, T* __restrict__ y,
+                                                                     float* __restrict__ rstd, int64_t rows, int cols,
+                                                                     int64_t stride, float eps) {
     constexpr int E = Pack16<T>::N;
-    const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * kRowsPerGroup + (threadIdx.x >> 6);
-    if (row >= rows) return;
+    constexpr int RPG = TPR == 256 ? 1 : 64 / TPR;  // rows per workgroup
+    __shared__ float red[4];
+    const int l = threadIdx.x % TPR;
+    const int64_t row = (int64_t)blockIdx.x * RPG + threadIdx.x / TPR;
+    const bool row_ok = row < rows;
     const T* xr = x + row * stride;
     T* yr = y + row * stride;
     Pack16<T> buf[NV];
-#pragma unroll
-    for (int u = 0; u < NV; ++u) {
-        const int c = (u * 64 + lane) * E;
-        if (c < cols) buf[u] = load16(xr + c);
-    }
     float ss = 0.f;
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-        const int c = (u * 64 + lane) * E;
-        if (c < cols) {
+        const int c = (u * TPR + l) * E;
+        if (row_ok && c < cols) buf[u] = load16(xr + c);
+    }
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int c = (u * TPR + l) * E;
+        if (row_ok && c < cols) {
 #pragma unroll
             for (int t = 0; t < E; ++t) {
                 const float f = (float)buf[u].v[t];
@@ -70,15 +94,15 @@ __global__ __launch_bounds__(64 * kRowsPerGroup) void srms_fwd_vec(const T* __re
             }
         }
     }
-    ss = wave_sum(ss);
+    ss = row_sum<TPR>(ss, red);
     const float rs = 1.0f / sqrtf(ss / (float)cols + eps);
-    if (lane == 0) rstd[row] = rs;
+    if (l == 0 && row_ok) rstd[row] = rs;
 #pragma unroll
     for (int u = 0; u < NV; ++u) forget(buf[u]);
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-        const int c = (u * 64 + lane) * E;
-        if (c < cols) {
+        const int c = (u * TPR + l) * E;
+        if (row_ok && c < cols) {
             Pack16<T> o;
 #pragma unroll
             for (int t = 0; t < E; ++t) o.v[t] = (T)((float)buf[u].v[t] * rs);
@@ -87,37 +111,39 @@ __global__ __launch_bounds__(64 * kRowsPerGroup) void srms_fwd_vec(const T* __re
     }
 }
 
-template <typename T, int NV>
-__global__ __launch_bounds__(64 * kRowsPerGroup) void srms_bwd_vec(const T* __restrict__ x, const T* __restrict__ dy,
-                                                    const float* __restrict__ rstd, T* __restrict__ dx,
-                                                    int64_t rows, int cols, int64_t stride) {
+template <typename T, int NV, int TPR>
+__global__ __launch_bounds__(TPR == 256 ? 256 : 64) void srms_bwd_vec(const T* __restrict__ x, const T* __restrict__ dy,
+                                                                     const float* __restrict__ rstd, T* __restrict__ dx,
+                                                                     int64_t rows, int cols, int64_t stride) {
     constexpr int E = Pack16<T>::N;
-    const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * kRowsPerGroup + (threadIdx.x >> 6);
-    if (row >= rows) return;
+    constexpr int RPG = TPR == 256 ? 1 : 64 / TPR;
+    __shared__ float red[4];
+    const int l = threadIdx.x % TPR;
+    const int64_t row = (int64_t)blockIdx.x * RPG + threadIdx.x / TPR;
+    const bool row_ok = row < rows;
     const T* xr = x + row * stride;
     const T* gr = dy + row * (int64_t)cols;  // dy and dx are dense (rows, cols)
     T* dr = dx + row * (int64_t)cols;
     Pack16<T> bx[NV], bg[NV];
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-        const int c = (u * 64 + lane) * E;
-        if (c < cols) {
+        const int c = (u * TPR + l) * E;
+        if (row_ok && c < cols) {
             bx[u] = load16(xr + c);
             bg[u] = load16(gr + c);
         }
     }
-    const float rs = rstd[row];
+    const float rs = row_ok ? rstd[row] : 0.f;
     float acc = 0.f;
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-        const int c = (u * 64 + lane) * E;
-        if (c < cols) {
+        const int c = (u * TPR + l) * E;
+        if (row_ok && c < cols) {
 #pragma unroll
             for (int t = 0; t < E; ++t) acc += ((float)bx[u].v[t] * rs) * (float)bg[u].v[t];
         }
     }
-    acc = wave_sum(acc);
+    acc = row_sum<TPR>(acc, red);
     const float m = acc / (float)cols;
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
@@ -126,8 +152,8 @@ __global__ __launch_bounds__(64 * kRowsPerGroup) void srms_bwd_vec(const T* __re
     }
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-        const int c = (u * 64 + lane) * E;
-        if (c < cols) {
+        const int c = (u * TPR + l) * E;
+        if (row_ok && c < cols) {
             Pack16<T> o;
 #pragma unroll
             for (int t = 0; t < E; ++t) {
@@ -140,15 +166,6 @@ __global__ __launch_bounds__(64 * kRowsPerGroup) void srms_bwd_vec(const T* __re
 }
 
 // ---- any cols / any alignment: one workgroup per row, scalar accesses ------
-__device__ __forceinline__ float block_sum_256(float v, float* red) {
-    v = wave_sum(v);
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-    __syncthreads();
-    const float t = red[0] + red[1] + red[2] + red[3];
-    __syncthreads();
-    return t;
-}
-
 template <typename T>
 __global__ __launch_bounds__(256) void srms_fwd_any(const T* __restrict__ x, T* __restrict__ y,
                                                     float* __restrict__ rstd, int64_t rows, int64_t cols,
@@ -190,23 +207,52 @@ __global__ __launch_bounds__(256) void srms_bwd_any(const T* __restrict__ x, con
 
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Shape of the register-resident kernels for a row of `chunks` 16-byte chunks: threads per row and
+// chunks per thread (0 = too wide).
+static void vec_shape(int64_t chunks, int* tpr, int* nv) {
+    *nv = 0;
+    if (chunks <= 32) {
+        *tpr = 4;
+        while (*tpr < chunks) *tpr *= 2;
+        *nv = 1;
+    } else if (chunks <= 64 * 16) {
+        *tpr = 64;
+        *nv = 1;
+        while (64 * *nv < chunks) *nv *= 2;
+    } else if (chunks <= 256 * 16) {
+        *tpr = 256;
+        *nv = 8;
+        while (256 * *nv < chunks) *nv *= 2;
+    }
+}
+
+#define LA_SRMS_DISPATCH(KERNEL, ...)                                                                      \
+    do {                                                                                                   \
+        const unsigned rpg = tpr == 256 ? 1u : 64u / (unsigned)tpr;                                        \
+        const dim3 grid((unsigned)((rows + rpg - 1) / rpg)), block(tpr == 256 ? 256 : 64);                 \
+        if (tpr == 4) hipLaunchKernelGGL((KERNEL<T, 1, 4>), grid, block, 0, st, __VA_ARGS__);              \
+        else if (tpr == 8) hipLaunchKernelGGL((KERNEL<T, 1, 8>), grid, block, 0, st, __VA_ARGS__);         \
+        else if (tpr == 16) hipLaunchKernelGGL((KERNEL<T, 1, 16>), grid, block, 0, st, __VA_ARGS__);       \
+        else if (tpr == 32) hipLaunchKernelGGL((KERNEL<T, 1, 32>), grid, block, 0, st, __VA_ARGS__);       \
+        else if (tpr == 64 && nv == 1) hipLaunchKernelGGL((KERNEL<T, 1, 64>), grid, block, 0, st, __VA_ARGS__);   \
+        else if (tpr == 64 && nv == 2) hipLaunchKernelGGL((KERNEL<T, 2, 64>), grid, block, 0, st, __VA_ARGS__);   \
+        else if (tpr == 64 && nv == 4) hipLaunchKernelGGL((KERNEL<T, 4, 64>), grid, block, 0, st, __VA_ARGS__);   \
+        else if (tpr == 64 && nv == 8) hipLaunchKernelGGL((KERNEL<T, 8, 64>), grid, block, 0, st, __VA_ARGS__);   \
+        else if (tpr == 64) hipLaunchKernelGGL((KERNEL<T, 16, 64>), grid, block, 0, st, __VA_ARGS__);      \
+        else if (nv == 8) hipLaunchKernelGGL((KERNEL<T, 8, 256>), grid, block, 0, st, __VA_ARGS__);        \
+        else hipLaunchKernelGGL((KERNEL<T, 16, 256>), grid, block, 0, st, __VA_ARGS__);                    \
+    } while (0)
+
 template <typename T>
 static int launch_fwd(const void* x, void* y, float* rstd, int64_t rows, int64_t cols, int64_t stride,
                       float eps, hipStream_t st) {
     constexpr int E = 16 / sizeof(T);
     const T* xp = static_cast<const T*>(x);
     T* yp = static_cast<T*>(y);
-    const bool vec = (cols % E == 0) && (stride % E == 0) && aligned16(x) && aligned16(y) && cols <= 64 * E * 16;
-    if (vec) {
-        const unsigned grid = (unsigned)((rows + kRowsPerGroup - 1) / kRowsPerGroup);
-        const int nv = (int)((cols + 64 * E - 1) / (64 * E));
-#define LA_FWD(NV) hipLaunchKernelGGL((srms_fwd_vec<T, NV>), dim3(grid), dim3(64 * kRowsPerGroup), 0, st, xp, yp, rstd, rows, (int)cols, stride, eps)
-        if (nv <= 1) LA_FWD(1);
-        else if (nv <= 2) LA_FWD(2);
-        else if (nv <= 4) LA_FWD(4);
-        else if (nv <= 8) LA_FWD(8);
-        else LA_FWD(16);
-#undef LA_FWD
+    int tpr = 0, nv = 0;
+    if ((cols % E == 0) && (stride % E == 0) && aligned16(x) && aligned16(y)) vec_shape(cols / E, &tpr, &nv);
+    if (nv) {
+        LA_SRMS_DISPATCH(srms_fwd_vec, xp, yp, rstd, rows, (int)cols, stride, eps);
     } else {
         hipLaunchKernelGGL((srms_fwd_any<T>), dim3((unsigned)rows), dim3(256), 0, st, xp, yp, rstd, rows, cols, stride, eps);
     }
@@ -220,22 +266,16 @@ static int launch_bwd(const void* x, const void* dy, const float* rstd, void* dx
     const T* xp = static_cast<const T*>(x);
     const T* gp = static_cast<const T*>(dy);
     T* dp = static_cast<T*>(dx);
-    const bool vec = (cols % E == 0) && (stride % E == 0) && aligned16(x) && aligned16(dy) && aligned16(dx) &&
-                     cols <= 64 * E * 8;
-    if (vec) {
-        const unsigned grid = (unsigned)((rows + kRowsPerGroup - 1) / kRowsPerGroup);
-        const int nv = (int)((cols + 64 * E - 1) / (64 * E));
-#define LA_BWD(NV) hipLaunchKernelGGL((srms_bwd_vec<T, NV>), dim3(grid), dim3(64 * kRowsPerGroup), 0, st, xp, gp, rstd, dp, rows, (int)cols, stride)
-        if (nv <= 1) LA_BWD(1);
-        else if (nv <= 2) LA_BWD(2);
-        else if (nv <= 4) LA_BWD(4);
-        else LA_BWD(8);
-#undef LA_BWD
+    int tpr = 0, nv = 0;
+    if ((cols % E == 0) && (stride % E == 0) && aligned16(x) && aligned16(dy) && aligned16(dx)) vec_shape(cols / E, &tpr, &nv);
+    if (nv) {
+        LA_SRMS_DISPATCH(srms_bwd_vec, xp, gp, rstd, dp, rows, (int)cols, stride);
     } else {
         hipLaunchKernelGGL((srms_bwd_any<T>), dim3((unsigned)rows), dim3(256), 0, st, xp, gp, rstd, dp, rows, cols, stride);
     }
     return (int)hipGetLastError();
 }
+#undef LA_SRMS_DISPATCH
 
 }  // namespace la
 

@@ -78,6 +78,27 @@ def test_odd_and_wide_rows(shape, dtype):
     assert_close(dx, dx_ref, atol=ATOL, rtol=RTOL)
 
 
+@pytest.mark.parametrize("cols", [8, 32, 40, 72, 136, 256, 264, 520, 1032, 2056, 4104, 8192, 8200, 16392, 32768])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_every_row_layout(cols, dtype):
+    """One width per kernel form: rows that share a wavefront (4, 8, 16, 32 lanes each), one wavefront per
+    row with 1 .. 16 chunks per lane, a four-wavefront workgroup per row; 37 rows, so the last wavefront
+    of the shared forms is partly empty."""
+    if cols * torch.empty((), dtype=dtype).element_size() > 65536:
+        pytest.skip("beyond the 64 KB row limit")
+    g = torch.Generator().manual_seed(cols)
+    x = torch.randn(37, cols, generator=g).to(dtype)
+    dy = torch.randn(37, cols, generator=g).to(dtype)
+    eps = 1.6e-5 if dtype == torch.float16 else 1e-6
+    y, dx = _run(x, dy)
+    y_ref, dx_ref = oracle.srmsnorm_fwd_bwd(x, dy, eps)
+    assert_close(y, y_ref, atol=ATOL, rtol=RTOL)
+    assert_close(dx, dx_ref, atol=ATOL, rtol=RTOL)
+    y64, dx64 = oracle.srmsnorm_fwd_bwd(x, dy, eps, torch.float64)
+    lim = 1e-6 if dtype == torch.float32 else (1e-3 if dtype == torch.float16 else 5e-3)
+    assert rel_norm(y, y64) < lim and rel_norm(dx, dx64) < lim
+
+
 def test_non_contiguous_input_and_row_limit():
     g = torch.Generator().manual_seed(4)
     x = torch.randn(6, 40, 512, generator=g).bfloat16().transpose(0, 1)
