@@ -104,8 +104,8 @@ def cpu_baseline(n_seq=10):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-sweep", action="store_true", help="skip the fwd/bwd split and the n sweep")
     ap.add_argument("--no-srms", action="store_true", help="skip the SRMSNorm timings")

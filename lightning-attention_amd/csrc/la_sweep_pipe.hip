@@ -201,8 +201,8 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
         if (DENSE) {
             // Plain tensors: one per-lane offset, rows >= n fall outside the buffer and the hardware
             // range check zeroes them.  Kept as its own code path because it is measurably faster
-            // (0.232 against 0.250 ms per launch at the headline shape) than the general form below,
-            // whose explicit row mask changes nothing in the memory traffic.
+            // (3 % per launch at b4 h32 n8192 d128) than the general form below, whose explicit row
+            // mask changes nothing in the memory traffic.
             const unsigned tok0 = (unsigned)(t * 64);
 #pragma unroll
             for (int u = 0; u < XC; ++u) {
