@@ -358,6 +358,25 @@ def test_full_size_against_block_recurrence_on_head_subset(n):
         check(got, (want_o,) + tuple(want_g), torch.bfloat16, "n=%d head (%d,%d)" % (n, bi, hi))
 
 
+def test_very_long_sequence_few_heads():
+    """n = 262144 (4096 blocks), b1 h2: the chunked walk at its longest; the slow-decay head against the
+    fp64 block recurrence, and no decay (a state that keeps growing) as well."""
+    b, h, n, d = 1, 2, 262144, 128
+    g = torch.Generator(device=DEV).manual_seed(31)
+    q, k, v, do = ((torch.randn(b, h, n, d, generator=g, device=DEV) * sc).bfloat16() for sc in (0.3, 0.3, 1.0, 1.0))
+    for s in (torch.tensor([0.5, 2.0 ** -8]).reshape(h, 1, 1), None):
+        qg, kg, vg = (t.clone().requires_grad_() for t in (q, k, v))
+        o = lightning_attn_func(qg, kg, vg, None if s is None else s.to(DEV))
+        o.backward(do)
+        torch.cuda.synchronize()
+        sub = [t[:, 1:2].float().cpu() for t in (q, k, v, do)]
+        ss = None if s is None else s[1:2]
+        want_o = oracle.block_recurrence_fwd(sub[0], sub[1], sub[2], ss, 64)
+        want_g = oracle.block_recurrence_bwd(sub[0], sub[1], sub[2], ss, sub[3], 64)
+        got = [t[:, 1:2] for t in (o.detach(), qg.grad, kg.grad, vg.grad)]
+        check(got, (want_o,) + tuple(want_g), torch.bfloat16, "n=262144 %s" % ("decay" if s is not None else "no decay"))
+
+
 def test_full_size_prefix_linearity_and_slicing():
     """Config 2 (b4 h32 n4096 d=e=128): causality (a prefix run reproduces the prefix bit for bit),
     linearity in v, and independence of batch/head slices."""
