@@ -37,7 +37,7 @@ enum {
     LA_E_NULLPTR = -1,     /* a required pointer is NULL                      */
     LA_E_SHAPE = -2,       /* a dimension is <= 0 or exceeds the index range  */
     LA_E_UNSUPPORTED = -3, /* head dims / dtype outside la_supported()        */
-    LA_E_WORKSPACE = -4,   /* workspace smaller than la_workspace_bytes()     */
+    LA_E_WORKSPACE = -4,   /* internal: scratch expected but absent            */
     LA_E_ALIGN = -5        /* a pointer or stride is not 16-byte aligned      */
 };
 
@@ -48,8 +48,14 @@ const char *la_error_string(int code);
  * d and e multiples of 8, 8 <= d,e <= 256 (<= 128 for float32).  Replaces the dimension gate
  * lightning_attn/ops/lightning_attn_interface.py:8-9,26 (is_support). */
 int la_supported(int64_t d, int64_t e, int dtype);
-/* Bytes of device scratch la_fwd (which=0) / la_bwd (which=1) need for these
- * shapes (0 when the single-sweep path is used). */
+/* Bytes of device scratch la_fwd (which=0) / la_bwd (which=1) can use for these shapes: 0 unless
+ * there are so few (batch, head) sequences that the walk over a long sequence is cut into chunks
+ * (the job of the reference's variant="parallel", lightning_attn/ops/triton/lightning_attn2_parallel.py:835-1072).
+ * The scratch then holds one d x e float state per chunk.  It is optional: with workspace == NULL,
+ * or fewer bytes than this, the chunks rebuild their incoming state by walking the blocks before
+ * them instead, which gives bit-identical results to the single walk and is several times slower
+ * for long sequences.  16-byte aligned; contents need not survive the call, and calls that follow
+ * each other on one stream may share it. */
 size_t la_workspace_bytes(int which, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype);
 
 /*

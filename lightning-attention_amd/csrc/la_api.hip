@@ -1,12 +1,15 @@
 // extern "C" entry points of the attention path (see include/lightning_attn_hip.h).
+#include <algorithm>
+
 #include "la_sweep_common.h"
 #include "lightning_attn_hip.h"
 
 namespace la {
 int sweep(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
-          bool reverse, hipStream_t st);
+          bool reverse, void* ws, size_t ws_bytes, hipStream_t st);
 int sweep2(const SweepIO& io0, const SweepIO& io1, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv,
-           int dtype, bool reverse, hipStream_t st);
+           int dtype, bool reverse, void* ws, size_t ws_bytes, hipStream_t st);
+size_t sweep_workspace_bytes(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int dtype);
 int sweep_f32(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
               int64_t n, int64_t dk, int64_t dv, bool reverse, hipStream_t st);
 
@@ -25,16 +28,22 @@ static SweepIO io(const Tensor& x, const Tensor& y, const Tensor& z, const Tenso
     return SweepIO{x.p, y.p, z.p, const_cast<void*>(out.p), x.l, y.l, z.l, out.l};
 }
 
+// caller's scratch memory (may be absent)
+struct Scratch {
+    void* p;
+    size_t bytes;
+};
+
 // one directional sweep at the element type named by dtype
 static int run(const Tensor& x, const Tensor& y, const Tensor& z, const Tensor& out, const float* s, int64_t bh, int64_t h,
-               int64_t n, int64_t dk, int64_t dv, int dtype, bool reverse, hipStream_t st) {
+               int64_t n, int64_t dk, int64_t dv, int dtype, bool reverse, const Scratch& ws, hipStream_t st) {
     if (dtype == LA_FP32) {
         // the float32 accuracy kernel takes plain (b, h, n, d) tensors only
         if (!is_dense(x, h, n, dk) || !is_dense(y, h, n, dk) || !is_dense(z, h, n, dv) || !is_dense(out, h, n, dv))
             return LA_E_UNSUPPORTED;
         return sweep_f32(x.p, y.p, z.p, const_cast<void*>(out.p), s, bh, h, n, dk, dv, reverse, st);
     }
-    return sweep(io(x, y, z, out), s, bh, h, n, dk, dv, dtype, reverse, st);
+    return sweep(io(x, y, z, out), s, bh, h, n, dk, dv, dtype, reverse, ws.p, ws.bytes, st);
 }
 
 static inline bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -62,7 +71,7 @@ static int check_tensor(const Tensor& t, int64_t b, int64_t h, int64_t n, int64_
 }
 
 static int fwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s, const Tensor& o, int64_t b, int64_t h,
-               int64_t n, int64_t d, int64_t e, int dtype, hipStream_t st) {
+               int64_t n, int64_t d, int64_t e, int dtype, const Scratch& ws, hipStream_t st) {
     int rc = check_dims(b, h, n, d, e, dtype);
     if (rc != LA_OK) return rc;
     if (b == 0 || n == 0) return LA_OK;  // nothing to do; empty tensors may carry null pointers
@@ -72,12 +81,12 @@ static int fwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s
         if (!ts[i]->p) return LA_E_NULLPTR;
     for (int i = 0; i < 4; ++i)
         if ((rc = check_tensor(*ts[i], b, h, n, cols[i], dtype)) != LA_OK) return rc;
-    return run(q, k, v, o, s, b * h, h, n, d, e, dtype, false, st);
+    return run(q, k, v, o, s, b * h, h, n, d, e, dtype, false, ws, st);
 }
 
 static int bwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s, const Tensor& dout, const Tensor& dq,
                const Tensor& dk, const Tensor& dv, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
-               hipStream_t st) {
+               const Scratch& ws, hipStream_t st) {
     int rc = check_dims(b, h, n, d, e, dtype);
     if (rc != LA_OK) return rc;
     if (b == 0 || n == 0) return LA_OK;
@@ -88,15 +97,16 @@ static int bwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s
     for (int i = 0; i < 7; ++i)
         if ((rc = check_tensor(*ts[i], b, h, n, cols[i], dtype)) != LA_OK) return rc;
     // dQ_i = sum_{j<=i} lam^(i-j) (dO_i . v_j) k_j
-    rc = run(dout, v, k, dq, s, b * h, h, n, e, d, dtype, false, st);
+    // (the launches follow each other on one stream, so they can all use the same scratch memory)
+    rc = run(dout, v, k, dq, s, b * h, h, n, e, d, dtype, false, ws, st);
     if (rc != LA_OK) return rc;
     // dK_j = sum_{i>=j} lam^(i-j) (v_j . dO_i) q_i   and   dV_j = sum_{i>=j} lam^(i-j) (k_j . q_i) dO_i
     // have the same shape when d == e: one launch, in which they share the reads of dO and q
     if (d == e && dtype != LA_FP32)
-        return sweep2(io(v, dout, q, dk), io(k, q, dout, dv), s, b * h, h, n, d, e, dtype, true, st);
-    rc = run(v, dout, q, dk, s, b * h, h, n, e, d, dtype, true, st);
+        return sweep2(io(v, dout, q, dk), io(k, q, dout, dv), s, b * h, h, n, d, e, dtype, true, ws.p, ws.bytes, st);
+    rc = run(v, dout, q, dk, s, b * h, h, n, e, d, dtype, true, ws, st);
     if (rc != LA_OK) return rc;
-    return run(k, q, dout, dv, s, b * h, h, n, d, e, dtype, true, st);
+    return run(k, q, dout, dv, s, b * h, h, n, d, e, dtype, true, ws, st);
 }
 }  // namespace la
 
@@ -125,44 +135,51 @@ extern "C" int la_supported(int64_t d, int64_t e, int dtype) {
 }
 
 extern "C" size_t la_workspace_bytes(int which, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype) {
-    (void)which; (void)b; (void)h; (void)n; (void)d; (void)e; (void)dtype;
-    return 0;
+    if (b <= 0 || h <= 0 || n <= 0 || !la_supported(d, e, dtype)) return 0;
+    using la::sweep_workspace_bytes;
+    const int64_t bh = b * h;
+    if (which == 0) return sweep_workspace_bytes(bh, n, d, e, 1, dtype);  // O = sweep(q, k, v)
+    // dQ = sweep(dO, v, k); then dK and dV, together when d == e
+    size_t need = sweep_workspace_bytes(bh, n, e, d, 1, dtype);
+    const size_t rest = d == e ? sweep_workspace_bytes(bh, n, d, e, 2, dtype)
+                               : std::max(sweep_workspace_bytes(bh, n, e, d, 1, dtype), sweep_workspace_bytes(bh, n, d, e, 1, dtype));
+    return std::max(need, rest);
 }
 
 extern "C" int la_fwd(const void* q, const void* k, const void* v, const float* s, void* o, int64_t b, int64_t h,
                       int64_t n, int64_t d, int64_t e, int dtype, void* workspace, size_t ws_bytes, void* stream) {
-    (void)workspace; (void)ws_bytes;
+    const la::Scratch ws = {workspace, workspace ? ws_bytes : 0};
     using la::dense;
     return la::fwd(dense(q, h, n, d), dense(k, h, n, d), dense(v, h, n, e), s, dense(o, h, n, e), b, h, n, d, e, dtype,
-                   static_cast<hipStream_t>(stream));
+                   ws, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int la_bwd(const void* q, const void* k, const void* v, const float* s, const void* dout, void* dq,
                       void* dk, void* dv, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
                       void* workspace, size_t ws_bytes, void* stream) {
-    (void)workspace; (void)ws_bytes;
+    const la::Scratch ws = {workspace, workspace ? ws_bytes : 0};
     using la::dense;
     return la::bwd(dense(q, h, n, d), dense(k, h, n, d), dense(v, h, n, e), s, dense(dout, h, n, e), dense(dq, h, n, d),
-                   dense(dk, h, n, d), dense(dv, h, n, e), b, h, n, d, e, dtype, static_cast<hipStream_t>(stream));
+                   dense(dk, h, n, d), dense(dv, h, n, e), b, h, n, d, e, dtype, ws, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int la_fwd_strided(const void* q, const void* k, const void* v, const float* s, void* o,
                               const int64_t* strides, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
                               void* workspace, size_t ws_bytes, void* stream) {
-    (void)workspace; (void)ws_bytes;
+    const la::Scratch ws = {workspace, workspace ? ws_bytes : 0};
     if (!strides) return LA_E_NULLPTR;
     using la::strided;
     return la::fwd(strided(q, strides), strided(k, strides + 3), strided(v, strides + 6), s, strided(o, strides + 9), b,
-                   h, n, d, e, dtype, static_cast<hipStream_t>(stream));
+                   h, n, d, e, dtype, ws, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int la_bwd_strided(const void* q, const void* k, const void* v, const float* s, const void* dout, void* dq,
                               void* dk, void* dv, const int64_t* strides, int64_t b, int64_t h, int64_t n, int64_t d,
                               int64_t e, int dtype, void* workspace, size_t ws_bytes, void* stream) {
-    (void)workspace; (void)ws_bytes;
+    const la::Scratch ws = {workspace, workspace ? ws_bytes : 0};
     if (!strides) return LA_E_NULLPTR;
     using la::strided;
     return la::bwd(strided(q, strides), strided(k, strides + 3), strided(v, strides + 6), s, strided(dout, strides + 9),
                    strided(dq, strides + 12), strided(dk, strides + 15), strided(dv, strides + 18), b, h, n, d, e, dtype,
-                   static_cast<hipStream_t>(stream));
+                   ws, static_cast<hipStream_t>(stream));
 }

@@ -569,38 +569,95 @@ static int launch_classic(const SweepPair& p, int dtype, bool reverse, hipStream
     return LA_E_UNSUPPORTED;
 }
 
-// x,y: (b,h,n,dk)  z,out: (b,h,n,dv), each with its own batch / head / token strides
-int sweep(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
-          bool reverse, hipStream_t st) {
-    SweepPair p;
-    p.nprod = 1;
-    p.wide = wide_columns(bh, dk, dv, 1) ? 1 : 0;
-    p.a[0] = make_args(io, s, bh, h, n, dk, dv);
-    if (p.wide) p.a[0].nslice = 1;
-    choose_chunks(p.a[0]);
-    p.a[1] = p.a[0];
+// With a workspace the pipelined kernel does not rebuild a chunk's incoming state with warm-up blocks:
+// it collects the states the chunks end with, scans them and starts every chunk from the result (three
+// launches; equally long chunks, up to 64 of them).  Number of chunks and bytes of workspace for a
+// launch of nprod sweeps, 0 bytes where the warm-up form is used.  LA_SWEEP_SCAN=0 keeps to the warm-up form.
+struct ScanPlan {
+    int nchunk, chunk_len;
+    size_t bytes;
+};
+static ScanPlan plan_scan(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, bool wide) {
+    ScanPlan pl = {1, 0, 0};
+    const char* off = getenv("LA_SWEEP_SCAN");
+    if (dk > 128 || (off && atoi(off) == 0)) return pl;
+    const char* env = getenv("LA_SWEEP_CHUNKS");
+    const int forced = env ? atoi(env) : 0;
+    const int64_t nblk = (n + 63) / 64, cus = num_cus();
+    const int64_t nslice = wide ? 1 : (dv + 63) / 64;
+    const int64_t wgs = (bh + 7) / 8 * 8 * nslice * nprod;
+    int64_t c = 1;
+    if (forced > 0) c = forced;
+    else if (wgs * 2 <= cus && nblk >= 128) {  // (shorter walks: three launches cost more than warm-up blocks)
+        c = cus / wgs;
+        if (c > nblk / 4) c = nblk / 4;  // at least four blocks per chunk
+    }
+    if (c > 64) c = 64;
+    if (c > nblk) c = nblk;
+    if (c < 2) return pl;
+    pl.chunk_len = (int)((nblk + c - 1) / c);
+    pl.nchunk = (int)((nblk + pl.chunk_len - 1) / pl.chunk_len);  // no empty chunk
+    if (pl.nchunk < 2 || bh * nprod * nslice > 65535) return ScanPlan{1, 0, 0};
+    pl.bytes = (size_t)(bh * nprod * nslice) * (size_t)(pl.nchunk - 1) * pipe_state_floats((int)dk, wide) * sizeof(float);
+    return pl;
+}
+
+// Workspace the pipelined kernel can use for one launch of nprod sweeps (0: none).
+size_t sweep_workspace_bytes(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int dtype) {
+    if (dtype != LA_BF16 && dtype != LA_FP16) return 0;
+    return plan_scan(bh, n, dk, dv, nprod, wide_columns(bh, dk, dv, nprod)).bytes;
+}
+
+static int launch_planned(SweepPair& p, int64_t bh, int64_t n, int64_t dk, int64_t dv, int dtype, bool reverse, void* ws,
+                          size_t ws_bytes, hipStream_t st) {
+    p.wide = wide_columns(bh, dk, dv, p.nprod) ? 1 : 0;
+    p.mode = kWarmUp;
+    p.chunk_len = 0;
+    p.state = nullptr;
+    for (int i = 0; i < p.nprod; ++i)
+        if (p.wide) p.a[i].nslice = 1;
+    const ScanPlan pl = plan_scan(bh, n, dk, dv, p.nprod, p.wide != 0);
+    if (pl.nchunk > 1 && ws && ws_bytes >= pl.bytes && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0) {
+        p.mode = kCollect;  // sweep_pipe runs the three launches
+        p.chunk_len = pl.chunk_len;
+        p.state = static_cast<float*>(ws);
+        for (int i = 0; i < p.nprod; ++i) {
+            p.a[i].nchunk = pl.nchunk;
+            for (int j = 0; j < 9; ++j) p.a[i].chunk_start[j] = 0;
+        }
+    } else {
+        choose_chunks(p.a[0], p.nprod);
+        for (int i = 1; i < p.nprod; ++i) {
+            p.a[i].nchunk = p.a[0].nchunk;
+            for (int j = 0; j < 9; ++j) p.a[i].chunk_start[j] = p.a[0].chunk_start[j];
+        }
+    }
+    if (p.nprod == 1) p.a[1] = p.a[0];
     if (dk <= 128) return sweep_pipe(p, dtype, reverse, st);  // pipelined kernel, la_sweep_pipe.hip
     return launch_classic(p, dtype, reverse, st);
 }
 
+// x,y: (b,h,n,dk)  z,out: (b,h,n,dv), each with its own batch / head / token strides
+int sweep(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
+          bool reverse, void* ws, size_t ws_bytes, hipStream_t st) {
+    SweepPair p;
+    p.nprod = 1;
+    p.a[0] = make_args(io, s, bh, h, n, dk, dv);
+    return launch_planned(p, bh, n, dk, dv, dtype, reverse, ws, ws_bytes, st);
+}
+
 // Two sweeps of the same shape and direction in one launch.
 int sweep2(const SweepIO& io0, const SweepIO& io1, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv,
-           int dtype, bool reverse, hipStream_t st) {
+           int dtype, bool reverse, void* ws, size_t ws_bytes, hipStream_t st) {
     if (getenv("LA_SWEEP_UNPAIRED")) {  // for measurements: two launches
-        const int rc = sweep(io0, s, bh, h, n, dk, dv, dtype, reverse, st);
-        return rc != LA_OK ? rc : sweep(io1, s, bh, h, n, dk, dv, dtype, reverse, st);
+        const int rc = sweep(io0, s, bh, h, n, dk, dv, dtype, reverse, ws, ws_bytes, st);
+        return rc != LA_OK ? rc : sweep(io1, s, bh, h, n, dk, dv, dtype, reverse, ws, ws_bytes, st);
     }
     SweepPair p;
     p.nprod = 2;
     p.a[0] = make_args(io0, s, bh, h, n, dk, dv);
     p.a[1] = make_args(io1, s, bh, h, n, dk, dv);
-    p.wide = wide_columns(bh, dk, dv, 2) ? 1 : 0;
-    if (p.wide) p.a[0].nslice = p.a[1].nslice = 1;
-    choose_chunks(p.a[0], 2);
-    p.a[1].nchunk = p.a[0].nchunk;
-    for (int i = 0; i < 9; ++i) p.a[1].chunk_start[i] = p.a[0].chunk_start[i];
-    if (dk <= 128) return sweep_pipe(p, dtype, reverse, st);
-    return launch_classic(p, dtype, reverse, st);
+    return launch_planned(p, bh, n, dk, dv, dtype, reverse, ws, ws_bytes, st);
 }
 
 }  // namespace la

@@ -99,10 +99,24 @@ struct SweepPair {
     SweepArgs a[2];
     int nprod;  // 1 or 2 sweeps; a[1] is unused when 1
     int wide;   // pipelined kernel only: a workgroup covers 128 instead of 64 columns of z / out
+    // Pipelined kernel only.  How a chunk's workgroup gets the state its chunk starts from:
+    //   kWarmUp   it walks the blocks before its chunk with the state update only (no workspace);
+    //   kCollect  first of three launches: every workgroup walks its own chunk, state update only, starting
+    //             from zero, and leaves the state it ends with in `state` (the last chunk has nothing to leave);
+    //   kApply    third launch: it starts from `state`, which the scan kernel run in between has turned
+    //             into the state at the start of each chunk.
+    // In the two latter modes the chunks are chunk_len blocks long (a[0].chunk_start is not used) and
+    // `state` holds, per (unit, sweep, slice), nchunk - 1 slots of the state waves' accumulators.
+    int mode;
+    int chunk_len;
+    float* state;
 };
 
 // Launches the single-barrier pipelined kernel (feature dim up to 128); defined in la_sweep_pipe.hip.
 // n, dk, dv, h, bh, nslice and the chunking must agree between the two sweeps of a pair.
+enum { kWarmUp = 0, kCollect = 1, kApply = 2 };
 int sweep_pipe(const SweepPair& p, int dtype, bool reverse, hipStream_t st);
+// Floats of one state slot of the pipelined kernel (dk padded to 64 or 128, 64 or 128 columns).
+inline size_t pipe_state_floats(int dk, bool wide) { return (size_t)(dk <= 64 ? 64 : 128) * (wide ? 128 : 64); }
 
 }  // namespace la

@@ -174,8 +174,21 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
     // Sequence chunking: this workgroup produces the blocks [it_first, it_end) of the walk.  It
     // first runs over the blocks before it_first with the state update only ("warm-up": y and z
     // are read, nothing is written) to rebuild the state its chunk starts from.
-    const int64_t it_first = a.chunk_start[chunk];
-    const int64_t it_end = a.chunk_start[chunk + 1];
+    // With a workspace (pair.mode != kWarmUp) the chunks are equally long and a workgroup walks its own
+    // chunk only: first with the state update alone, from zero, to leave the state it ends with
+    // (kCollect), then - a scan kernel having combined those into the state at the start of every
+    // chunk - for good, from that state (kApply).
+    const int mode = pair.mode;
+    const int nchunk = pair.a[0].nchunk;
+    if (mode == kCollect && chunk == nchunk - 1) return;  // nobody needs the state after the last chunk
+    const int64_t cbeg = mode == kWarmUp ? (int64_t)a.chunk_start[chunk] : min((int64_t)chunk * pair.chunk_len, nblk);
+    const int64_t cend = mode == kWarmUp ? (int64_t)a.chunk_start[chunk + 1] : min((int64_t)(chunk + 1) * pair.chunk_len, nblk);
+    const int64_t it0 = mode == kWarmUp ? 0 : cbeg;           // first block this workgroup walks
+    const int64_t it_first = mode == kCollect ? cend : cbeg;  // first block whose output it produces
+    const int64_t it_end = cend;
+    // the state slot of this workgroup's chunk: [unit][sweep][slice][chunk 0 .. nchunk-2][state waves' accumulators]
+    constexpr size_t SF = (size_t)4 * NH * KT * 64 * 4;
+    float* const slot0 = pair.state + ((((size_t)unit * nprod + sub % nprod) * nslice + slice) * (size_t)(nchunk - 1)) * SF;
 
     u32x4 xrA[XC], yrA[XC], zrA[ZC], xrB[XC], yrB[XC], zrB[ZC];
 
@@ -197,7 +210,7 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
         const bool valid = b < it_end, need_x = valid && b >= it_first;
         // the z slice that travels with this block's x / y tiles
         const int64_t bz = b - ZLAG, tz = REVERSE ? nblk - 1 - bz : bz;
-        const bool validz = bz >= 0 && bz < it_end;
+        const bool validz = bz >= it0 && bz < it_end;
         if (DENSE) {
             // Plain tensors: one per-lane offset, rows >= n fall outside the buffer and the hardware
             // range check zeroes them.  Kept as its own code path because it is measurably faster
@@ -476,7 +489,7 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
                         *reinterpret_cast<V4*>(smem + oq + (16 * i4 * ZS + 16 * h) * E) = o;
                     }
             }
-            if (have_next) {
+            if (have_next || mode == kCollect) {
                 // state = lam^64 state + y^T (z * Lupd)
                 V8 ay[KT][2];
 #pragma unroll
@@ -518,7 +531,7 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
     // The two kinds of waves run separate copies of the loop (one barrier per iteration in each),
     // so that neither carries the other's registers.
     auto walk = [&](auto role) __attribute__((always_inline)) {
-        int64_t it = 0;
+        int64_t it = it0;
         for (; it + 1 < it_end; it += 2) {
             iteration(role, it, xrA, yrA, zrA);
             iteration(role, it + 1, xrB, yrB, zrB);
@@ -539,14 +552,15 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
     // runs, whatever the second one needs of the values computed before this point - which must
     // therefore not include the score waves' prefetch registers.
     if (!state_role) {
-        load_block(0, xrA, yrA, zrA);
-        load_block(1, xrB, yrB, zrB);
-        stage_block(0, NH == 1 ? 0 : 1, xrA, yrA, zrA, 0, false);
-        load_block(2, xrA, yrA, zrA);
-        stage_block(1, NH == 1 ? 1 : 0, xrB, yrB, zrB, 0, false);
-        load_block(3, xrB, yrB, zrB);
+        const int b0 = (int)((unsigned)it0 % 3u), b1 = b0 == 2 ? 0 : b0 + 1;
+        load_block(it0, xrA, yrA, zrA);
+        load_block(it0 + 1, xrB, yrB, zrB);
+        stage_block(b0, NH == 1 ? b0 : (int)((it0 + 1) & 1), xrA, yrA, zrA, 0, false);
+        load_block(it0 + 2, xrA, yrA, zrA);
+        stage_block(b1, NH == 1 ? b1 : (int)(it0 & 1), xrB, yrB, zrB, 0, false);
+        load_block(it0 + 3, xrB, yrB, zrB);
         __syncthreads();
-        if (it_first == 0) score_block(0, 0);
+        if (it0 >= it_first && it0 < it_end) score_block(b0, (int)(it0 & 1));
         __syncthreads();
         walk(std::false_type{});
         flush_last();
@@ -556,11 +570,23 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
         // The state waves are the critical path and every SIMD holds one wave of each kind: when both
         // have an instruction ready (right after the barrier all eight waves go for LDS), theirs goes first.
         __builtin_amdgcn_s_setprio(1);
+        // this lane's part of a state slot: [wave][slab][tile][lane] accumulator quartets
+        const size_t lane_slot = ((size_t)w * NH * KT * 64 + lane) * 4;
+        const bool resume = mode == kApply && chunk > 0;
+        const float* const src = slot0 + (size_t)(chunk - 1) * SF + lane_slot;
 #pragma unroll
         for (int h = 0; h < NH; ++h)
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt) st[h][kt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            for (int kt = 0; kt < KT; ++kt)
+                st[h][kt] = resume ? *reinterpret_cast<const f32x4*>(src + (size_t)(h * KT + kt) * 256) : (f32x4){0.f, 0.f, 0.f, 0.f};
         walk(std::true_type{});
+        if (mode == kCollect) {
+            float* const dst = slot0 + (size_t)chunk * SF + lane_slot;
+#pragma unroll
+            for (int h = 0; h < NH; ++h)
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<f32x4*>(dst + (size_t)(h * KT + kt) * 256) = st[h][kt];
+        }
     }
 }
 
@@ -604,11 +630,55 @@ static int launch_dir(const SweepPair& pair, hipStream_t st) {
 #undef LA_GO2
 }
 
-int sweep_pipe(const SweepPair& p, int dtype, bool reverse, hipStream_t st) {
-    if (p.a[0].dk > 128 || p.nprod < 1 || p.nprod > 2) return LA_E_UNSUPPORTED;
+// Between kCollect and kApply: turns the states the chunks end with (each computed from zero) into the
+// states they start from.  Slot c holds S_loc[c] on entry and S_in[c + 1] = lam^(64 len_c) S_in[c] + S_loc[c]
+// on exit (S_in[0] = 0).  One thread per accumulator quartet, chunks in order; the layout inside a slot
+// does not matter.
+__global__ __launch_bounds__(256) void la_state_scan_kernel(float* state, const float* s, int h, int sets_per_unit,
+                                                           int nchunk, int chunk_len, int64_t nblk, int quartets) {
+    const int q = blockIdx.x * 256 + threadIdx.x;  // quartet within the slot
+    const int64_t set = blockIdx.y;                // (unit, sweep, slice)
+    if (q >= quartets) return;
+    const float rate = s ? s[(set / sets_per_unit) % h] : 0.f;
+    f32x4* slot = reinterpret_cast<f32x4*>(state) + set * (int64_t)(nchunk - 1) * quartets + q;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c + 1 < nchunk; ++c) {
+        const int64_t b0 = min((int64_t)c * chunk_len, nblk), b1 = min((int64_t)(c + 1) * chunk_len, nblk);
+        const float f = s ? expf(-rate * 64.f * (float)(b1 - b0)) : 1.f;
+        acc = acc * f + slot[(int64_t)c * quartets];
+        slot[(int64_t)c * quartets] = acc;
+    }
+}
+
+static int launch_any(const SweepPair& p, int dtype, bool reverse, hipStream_t st) {
     if (dtype == LA_BF16) return reverse ? launch_dir<__bf16, true>(p, st) : launch_dir<__bf16, false>(p, st);
     if (dtype == LA_FP16) return reverse ? launch_dir<_Float16, true>(p, st) : launch_dir<_Float16, false>(p, st);
     return LA_E_UNSUPPORTED;
+}
+
+int sweep_pipe(const SweepPair& p, int dtype, bool reverse, hipStream_t st) {
+    const SweepArgs& a = p.a[0];
+    if (a.dk > 128 || p.nprod < 1 || p.nprod > 2) return LA_E_UNSUPPORTED;
+    if (p.mode == kWarmUp || a.nchunk <= 1) {
+        SweepPair q = p;
+        q.mode = kWarmUp;
+        return launch_any(q, dtype, reverse, st);
+    }
+    if (!p.state || p.chunk_len < 1) return LA_E_WORKSPACE;
+    // three launches: local end states, their scan, the walk proper
+    SweepPair q = p;
+    q.mode = kCollect;
+    int rc = launch_any(q, dtype, reverse, st);
+    if (rc != LA_OK) return rc;
+    const int quartets = (int)(pipe_state_floats(a.dk, p.wide != 0) / 4);
+    const int sets_per_unit = p.nprod * a.nslice;
+    const int64_t nblk = (a.n + 63) / 64;
+    hipLaunchKernelGGL(la_state_scan_kernel, dim3((unsigned)((quartets + 255) / 256), (unsigned)(a.bh * sets_per_unit)),
+                       dim3(256), 0, st, p.state, a.s, a.h, sets_per_unit, a.nchunk, p.chunk_len, nblk, quartets);
+    rc = (int)hipGetLastError();
+    if (rc != LA_OK) return rc;
+    q.mode = kApply;
+    return launch_any(q, dtype, reverse, st);
 }
 
 }  // namespace la

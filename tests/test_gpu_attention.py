@@ -227,11 +227,12 @@ def test_wide_features_are_split_by_the_interface():
 
 @pytest.mark.parametrize("b, h, n, d, e", [(1, 2, 4096, 128, 64), (2, 3, 1000, 64, 128), (1, 1, 1500, 192, 72)])
 def test_sequence_chunking_is_exact(b, h, n, d, e, monkeypatch):
-    """Few sequences: the walk is cut into chunks whose workgroups rebuild their incoming state
-    (the chunk-parallel path).  Every chunk count must give bit-identical results, and they must
-    match the oracle."""
+    """Few sequences: the walk is cut into chunks whose workgroups rebuild their incoming state with
+    warm-up blocks (the chunk-parallel path without a workspace, LA_SWEEP_SCAN=0).  Every chunk count
+    must give bit-identical results, and they must match the oracle."""
     q, k, v, do = make_inputs(b, h, n, d, e, torch.bfloat16, 1.0, seed=n)
     s = _build_slope_tensor(h)
+    monkeypatch.setenv("LA_SWEEP_SCAN", "0")
     outs = {}
     for chunks in ("1", "2", "3", "8", None):  # None = the library's own choice
         if chunks is None:
@@ -240,11 +241,35 @@ def test_sequence_chunking_is_exact(b, h, n, d, e, monkeypatch):
             monkeypatch.setenv("LA_SWEEP_CHUNKS", chunks)
         outs[chunks] = run_hip(q, k, v, s, do)
     monkeypatch.delenv("LA_SWEEP_CHUNKS", raising=False)
+    monkeypatch.delenv("LA_SWEEP_SCAN", raising=False)
     for chunks in ("2", "3", "8", None):
         for a, c in zip(outs["1"], outs[chunks]):
             assert torch.equal(a, c), chunks
     want = oracle.linear_attn_fwd_bwd(q, k, v, s, do, torch.float32)
     check(outs[None], want, torch.bfloat16, "chunked %s" % ((b, h, n, d, e),))
+
+
+@pytest.mark.parametrize("b, h, n, d, e", [(1, 2, 4096, 128, 64), (2, 3, 1000, 64, 128), (1, 2, 2100, 128, 128), (1, 1, 1500, 96, 72)])
+@pytest.mark.parametrize("decay", [True, False])
+def test_chunk_states_by_scan(b, h, n, d, e, decay, monkeypatch):
+    """With a workspace (the Python operators always pass one) the d <= 128 kernel starts every chunk from
+    a scanned state instead of rebuilding it: three launches, up to 64 chunks.  The state sums are taken
+    in another order, so results agree with the single walk to rounding, not bit for bit."""
+    q, k, v, do = make_inputs(b, h, n, d, e, torch.bfloat16, 1.0, seed=n + d)
+    s = _build_slope_tensor(h) if decay else None
+    monkeypatch.setenv("LA_SWEEP_CHUNKS", "1")
+    one = run_hip(q, k, v, s, do)
+    want = oracle.linear_attn_fwd_bwd(q, k, v, s, do, torch.float32)
+    for chunks in ("2", "3", "7", "16", "64", None):
+        if chunks is None:
+            monkeypatch.delenv("LA_SWEEP_CHUNKS", raising=False)
+        else:
+            monkeypatch.setenv("LA_SWEEP_CHUNKS", chunks)
+        got = run_hip(q, k, v, s, do)
+        for name, a, c in zip(("o", "dq", "dk", "dv"), got, one):
+            assert rel_norm(a, c) < 5e-4, (chunks, name, rel_norm(a, c))
+        check(got, want, torch.bfloat16, "scan, %s chunks %s" % (chunks, (b, h, n, d, e)))
+    monkeypatch.delenv("LA_SWEEP_CHUNKS", raising=False)
 
 
 @pytest.mark.parametrize("chunks", ["2", "5"])
@@ -256,14 +281,19 @@ def test_chunked_walk_on_projection_layout(chunks, monkeypatch):
     q, k = ((torch.randn(b, n, h, d, generator=g) * 0.7).bfloat16().to(DEV).transpose(1, 2) for _ in range(2))
     v, do = (torch.randn(b, n, h, e, generator=g).bfloat16().to(DEV).transpose(1, 2) for _ in range(2))
     s = _build_slope_tensor(h)
+    monkeypatch.setenv("LA_SWEEP_SCAN", "0")  # warm-up chunks: bit-identical to the single walk
     monkeypatch.setenv("LA_SWEEP_CHUNKS", chunks)
     got = run_hip(q.detach(), k.detach(), v.detach(), s, do)  # fresh leaves for every call
     got_plain = run_hip(q.contiguous(), k.contiguous(), v.contiguous(), s, do.contiguous())
     monkeypatch.setenv("LA_SWEEP_CHUNKS", "1")
     got_one = run_hip(q.detach(), k.detach(), v.detach(), s, do)
+    monkeypatch.delenv("LA_SWEEP_SCAN", raising=False)
+    monkeypatch.setenv("LA_SWEEP_CHUNKS", chunks)
+    got_scan = run_hip(q.detach(), k.detach(), v.detach(), s, do)  # the same chunks from scanned states
     monkeypatch.delenv("LA_SWEEP_CHUNKS", raising=False)
-    for a, c, one in zip(got, got_plain, got_one):
+    for a, c, one, sc in zip(got, got_plain, got_one, got_scan):
         assert torch.equal(a, c) and torch.equal(a, one)
+        assert rel_norm(sc, a) < 5e-4
     want = oracle.linear_attn_fwd_bwd(q.cpu(), k.cpu(), v.cpu(), s, do.cpu(), torch.float32)
     check(got, want, torch.bfloat16, "chunked token-major")
 
@@ -276,6 +306,7 @@ def test_paired_backward_launch_matches_separate_launches(b, h, n, d, monkeypatc
     them one after the other.  Same numbers, bit for bit, also when the walk is cut into chunks."""
     q, k, v, do = make_inputs(b, h, n, d, d, torch.bfloat16, 1.0, seed=d + n)
     s = _build_slope_tensor(h)
+    monkeypatch.setenv("LA_SWEEP_SCAN", "0")  # (scanned chunk states agree to rounding only)
     got = {}
     for mode, env in (("narrow", {"LA_SWEEP_WIDE": "0"}), ("wide", {"LA_SWEEP_WIDE": "1"}),
                       ("wide chunked", {"LA_SWEEP_WIDE": "1", "LA_SWEEP_CHUNKS": "3"}), ("separate", {"LA_SWEEP_UNPAIRED": "1"})):
@@ -284,7 +315,7 @@ def test_paired_backward_launch_matches_separate_launches(b, h, n, d, monkeypatc
         for name, value in env.items():
             monkeypatch.setenv(name, value)
         got[mode] = run_hip(q, k, v, s, do)
-    for name in ("LA_SWEEP_WIDE", "LA_SWEEP_CHUNKS", "LA_SWEEP_UNPAIRED"):
+    for name in ("LA_SWEEP_WIDE", "LA_SWEEP_CHUNKS", "LA_SWEEP_UNPAIRED", "LA_SWEEP_SCAN"):
         monkeypatch.delenv(name, raising=False)
     for mode in ("narrow", "wide", "wide chunked"):
         for a, c in zip(got[mode], got["separate"]):

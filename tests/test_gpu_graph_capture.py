@@ -31,12 +31,16 @@ def test_forward_backward_replay_from_a_graph(b, h, n, d):
     o, dq, dk, dv = (torch.empty_like(q) for _ in range(4))
     s = _build_slope_tensor(h).to(dev).reshape(h).contiguous()
 
+    # the caller's scratch memory (chunk states, where the library cuts the sequence): allocated once, outside
+    ws_bytes = max(L.la_workspace_bytes(0, b, h, n, d, d, code), L.la_workspace_bytes(1, b, h, n, d, d, code))
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+
     def enqueue():
         st = _lib.stream_ptr(dev)
         _lib.check(L.la_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr(), o.data_ptr(), b, h, n, d, d, code,
-                            None, 0, st), "la_fwd")
+                            ws.data_ptr(), ws_bytes, st), "la_fwd")
         _lib.check(L.la_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr(), do.data_ptr(), dq.data_ptr(),
-                            dk.data_ptr(), dv.data_ptr(), b, h, n, d, d, code, None, 0, st), "la_bwd")
+                            dk.data_ptr(), dv.data_ptr(), b, h, n, d, d, code, ws.data_ptr(), ws_bytes, st), "la_bwd")
 
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
