@@ -37,7 +37,16 @@ def test_host_only_entry_points():
         assert L.la_supported(d, e, dt) == want, (d, e, dt)
     assert L.la_error_string(0) == b"success"
     assert b"NULL" in L.la_error_string(-1)
-    assert L.la_workspace_bytes(0, 4, 32, 8192, 128, 128, 0) >= 0
+    # scratch for the chunked walk: none when the sequences fill the chip, short walks, wide dims or float32;
+    # otherwise one d x e (padded) float state per chunk but the last, per sequence and column slice
+    assert L.la_workspace_bytes(0, 4, 32, 8192, 128, 128, 0) == 0
+    assert L.la_workspace_bytes(1, 4, 32, 8192, 128, 128, 0) == 0
+    assert L.la_workspace_bytes(0, 1, 8, 2048, 128, 128, 0) == 0
+    assert L.la_workspace_bytes(0, 1, 8, 8192, 192, 192, 0) == 0
+    assert L.la_workspace_bytes(0, 1, 8, 8192, 128, 128, 2) == 0
+    need = L.la_workspace_bytes(0, 1, 8, 8192, 128, 128, 0)
+    assert need > 0 and need % (128 * 64 * 4) == 0 and need <= 8 * 2 * 63 * 128 * 64 * 4
+    assert L.la_workspace_bytes(1, 1, 8, 8192, 128, 128, 0) >= need
     # argument errors are reported before any launch, so they are testable without a device
     assert L.la_fwd(None, None, None, None, None, 1, 1, 64, 64, 64, 0, None, 0, None) == -1
     buf = ctypes.create_string_buffer(64)
