@@ -549,6 +549,7 @@ static bool wide_columns(int64_t bh, int64_t dk, int64_t dv, int nprod) {
     if (dk > 128 || dv <= 64 || dv > 128) return false;
     const char* env = getenv("LA_SWEEP_WIDE");
     if (env) return atoi(env) != 0;
+    if (dk <= 64) return false;  // the 128-column form pads the feature dim to 128
     const int64_t cus = num_cus(), wide = (bh + 7) / 8 * 8 * nprod, narrow = 2 * wide;
     if (narrow <= cus) return false;  // every 64-column workgroup gets a CU of its own
     return (wide + cus - 1) / cus * 5 < (narrow + cus - 1) / cus * 4;

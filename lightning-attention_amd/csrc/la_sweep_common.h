@@ -116,7 +116,9 @@ struct SweepPair {
 // n, dk, dv, h, bh, nslice and the chunking must agree between the two sweeps of a pair.
 enum { kWarmUp = 0, kCollect = 1, kApply = 2 };
 int sweep_pipe(const SweepPair& p, int dtype, bool reverse, hipStream_t st);
-// Floats of one state slot of the pipelined kernel (dk padded to 64 or 128, 64 or 128 columns).
-inline size_t pipe_state_floats(int dk, bool wide) { return (size_t)(dk <= 64 ? 64 : 128) * (wide ? 128 : 64); }
+// Floats of one state slot of the pipelined kernel (dk padded to 64 or 128, 64 or 128 columns): must
+// agree with the kernel's own SF.
+// (the 128-column form exists for the 128-wide feature tile only)
+inline size_t pipe_state_floats(int dk, bool wide) { return (size_t)(dk <= 64 && !wide ? 64 : 128) * (wide ? 128 : 64); }
 
 }  // namespace la

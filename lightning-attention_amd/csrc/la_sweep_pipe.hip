@@ -602,6 +602,8 @@ static int launch_one(const SweepPair& pair, hipStream_t st) {
         if (e != hipSuccess) return (int)e;
     }
     const int units8 = (a.bh + 7) / 8 * 8;
+    // the state slots the host sized must be the ones this instantiation reads and writes
+    if (pair.mode != kWarmUp && pipe_state_floats(a.dk, pair.wide != 0) != (size_t)4 * NH * (DKP / 16) * 64 * 4) return LA_E_WORKSPACE;
     const unsigned grid = (unsigned)(units8 * a.nslice * a.nchunk * pair.nprod);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, st, pair);
     return (int)hipGetLastError();

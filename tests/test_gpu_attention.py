@@ -249,7 +249,8 @@ def test_sequence_chunking_is_exact(b, h, n, d, e, monkeypatch):
     check(outs[None], want, torch.bfloat16, "chunked %s" % ((b, h, n, d, e),))
 
 
-@pytest.mark.parametrize("b, h, n, d, e", [(1, 2, 4096, 128, 64), (2, 3, 1000, 64, 128), (1, 2, 2100, 128, 128), (1, 1, 1500, 96, 72)])
+@pytest.mark.parametrize("b, h, n, d, e", [(1, 2, 4096, 128, 64), (2, 3, 1000, 64, 128), (1, 2, 2100, 128, 128), (1, 1, 1500, 96, 72),
+                                           (3, 1, 831, 16, 128), (1, 2, 900, 64, 64)])
 @pytest.mark.parametrize("decay", [True, False])
 def test_chunk_states_by_scan(b, h, n, d, e, decay, monkeypatch):
     """With a workspace (the Python operators always pass one) the d <= 128 kernel starts every chunk from
@@ -260,16 +261,22 @@ def test_chunk_states_by_scan(b, h, n, d, e, decay, monkeypatch):
     monkeypatch.setenv("LA_SWEEP_CHUNKS", "1")
     one = run_hip(q, k, v, s, do)
     want = oracle.linear_attn_fwd_bwd(q, k, v, s, do, torch.float32)
-    for chunks in ("2", "3", "7", "16", "64", None):
-        if chunks is None:
-            monkeypatch.delenv("LA_SWEEP_CHUNKS", raising=False)
+    for wide in (None, "0", "1"):  # the library's choice, 64-column, 128-column workgroups
+        if wide is None:
+            monkeypatch.delenv("LA_SWEEP_WIDE", raising=False)
         else:
-            monkeypatch.setenv("LA_SWEEP_CHUNKS", chunks)
-        got = run_hip(q, k, v, s, do)
-        for name, a, c in zip(("o", "dq", "dk", "dv"), got, one):
-            assert rel_norm(a, c) < 5e-4, (chunks, name, rel_norm(a, c))
-        check(got, want, torch.bfloat16, "scan, %s chunks %s" % (chunks, (b, h, n, d, e)))
+            monkeypatch.setenv("LA_SWEEP_WIDE", wide)
+        for chunks in ("2", "3", "7", "16", "64", None):
+            if chunks is None:
+                monkeypatch.delenv("LA_SWEEP_CHUNKS", raising=False)
+            else:
+                monkeypatch.setenv("LA_SWEEP_CHUNKS", chunks)
+            got = run_hip(q, k, v, s, do)
+            for name, a, c in zip(("o", "dq", "dk", "dv"), got, one):
+                assert rel_norm(a, c) < 5e-4, (wide, chunks, name, rel_norm(a, c))
+            check(got, want, torch.bfloat16, "scan, wide %s, %s chunks %s" % (wide, chunks, (b, h, n, d, e)))
     monkeypatch.delenv("LA_SWEEP_CHUNKS", raising=False)
+    monkeypatch.delenv("LA_SWEEP_WIDE", raising=False)
 
 
 @pytest.mark.parametrize("chunks", ["2", "5"])
