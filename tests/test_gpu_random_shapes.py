@@ -1,5 +1,6 @@
-"""Seeded random walk over shapes, dtypes, layouts and launch modes (sequence chunks, 64- / 128-column
-workgroups, paired / separate dK + dV launches), each case against the naive oracle."""
+"""Seeded random walk over shapes, dtypes, layouts and launch modes (sequence chunks from scanned states or
+with warm-up blocks, 64- / 128-column workgroups, paired / separate dK + dV launches), each case against the
+naive oracle."""
 import os
 import random
 import sys
@@ -17,17 +18,17 @@ from oracle import linear_attn_oracle as oracle  # noqa: E402
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
-KNOBS = ("LA_SWEEP_WIDE", "LA_SWEEP_CHUNKS", "LA_SWEEP_UNPAIRED")
+KNOBS = ("LA_SWEEP_WIDE", "LA_SWEEP_CHUNKS", "LA_SWEEP_UNPAIRED", "LA_SWEEP_SCAN")
 
 
 def _rel(a, r):
     return ((a.float().cpu() - r.float()).norm() / (r.float().norm() + 1e-30)).item()
 
 
-@pytest.mark.parametrize("seed", [101, 202, 303])
+@pytest.mark.parametrize("seed", [101, 202, 303, 404, 505])
 def test_random_cases_match_the_oracle(seed, monkeypatch):
     rnd = random.Random(seed)
-    for case in range(14):
+    for case in range(20):
         b, h = rnd.randint(1, 3), rnd.randint(1, 9)
         n = rnd.choice([1, 2, 63, 64, 65, 127, 128, 129, 300, 513, 777, 1000, rnd.randint(1, 1200)])
         d = 8 * rnd.randint(1, 32)
@@ -38,8 +39,10 @@ def test_random_cases_match_the_oracle(seed, monkeypatch):
         env = {}
         if rnd.random() < 0.6:
             env["LA_SWEEP_WIDE"] = rnd.choice(["0", "1"])
-        if rnd.random() < 0.5:
-            env["LA_SWEEP_CHUNKS"] = str(rnd.randint(1, 5))
+        if rnd.random() < 0.6:
+            env["LA_SWEEP_CHUNKS"] = str(rnd.choice([1, 2, 3, 4, 5, 9, 17, 40, 64]))
+        if rnd.random() < 0.3:
+            env["LA_SWEEP_SCAN"] = "0"
         if rnd.random() < 0.2:
             env["LA_SWEEP_UNPAIRED"] = "1"
         for name in KNOBS:
