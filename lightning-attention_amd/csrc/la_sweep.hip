@@ -545,13 +545,19 @@ static void choose_chunks(SweepArgs& a, int nprod = 1) {
 // as there are workgroups enough.  A 128-column workgroup takes about 1.25 times as long as a
 // 64-column one, and there are half as many: compare the rounds of workgroups the chip has to run.
 // LA_SWEEP_WIDE=0 / 1 overrides the choice.
-static bool wide_columns(int64_t bh, int64_t dk, int64_t dv, int nprod) {
+static bool wide_columns(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod) {
     if (dk > 128 || dv <= 64 || dv > 128) return false;
     const char* env = getenv("LA_SWEEP_WIDE");
     if (env) return atoi(env) != 0;
     if (dk <= 64) return false;  // the 128-column form pads the feature dim to 128
     const int64_t cus = num_cus(), wide = (bh + 7) / 8 * 8 * nprod, narrow = 2 * wide;
-    if (narrow <= cus) return false;  // every 64-column workgroup gets a CU of its own
+    if (narrow <= cus) {
+        // Every 64-column workgroup gets a CU of its own.  With so few of them that a long walk is cut
+        // into chunks anyway, rather half as many workgroups of 128 columns and twice the chunks
+        // (b1 h32 n8192 fwd+bwd 0.28 against 0.34 ms, b1 h4 n65536 0.46 against 0.62).
+        const char* off = getenv("LA_SWEEP_SCAN");
+        return narrow * 2 <= cus && (n + 63) / 64 >= 128 && !(off && atoi(off) == 0);
+    }
     return (wide + cus - 1) / cus * 5 < (narrow + cus - 1) / cus * 4;
 }
 
@@ -606,12 +612,12 @@ static ScanPlan plan_scan(int64_t bh, int64_t n, int64_t dk, int64_t dv, int npr
 // Workspace the pipelined kernel can use for one launch of nprod sweeps (0: none).
 size_t sweep_workspace_bytes(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int dtype) {
     if (dtype != LA_BF16 && dtype != LA_FP16) return 0;
-    return plan_scan(bh, n, dk, dv, nprod, wide_columns(bh, dk, dv, nprod)).bytes;
+    return plan_scan(bh, n, dk, dv, nprod, wide_columns(bh, n, dk, dv, nprod)).bytes;
 }
 
 static int launch_planned(SweepPair& p, int64_t bh, int64_t n, int64_t dk, int64_t dv, int dtype, bool reverse, void* ws,
                           size_t ws_bytes, hipStream_t st) {
-    p.wide = wide_columns(bh, dk, dv, p.nprod) ? 1 : 0;
+    p.wide = wide_columns(bh, n, dk, dv, p.nprod) ? 1 : 0;
     p.mode = kWarmUp;
     p.chunk_len = 0;
     p.state = nullptr;
