@@ -20,6 +20,11 @@
 //   - the output tile of block `it`, which the state waves write over the z columns they
 //     alone read and which leaves for memory as whole row segments when that z slot is
 //     refilled one iteration later.
+// With few (batch, head) sequences the walk is cut into chunks, one workgroup each.  A chunk's
+// incoming state comes either from warm-up blocks (the workgroup first walks everything before its
+// chunk with the state update alone) or, given a workspace, from a scan: the same kernel run once in
+// "collect" mode (every chunk's own blocks, state update alone, end state written out), a small scan
+// kernel, and the kernel again in "apply" mode (state read in, the chunk walked for good).
 // The chip runs this kernel at its socket power limit, so what counts is the work per output
 // element (LDS traffic above all), not the length of any dependency chain: hence the 128-column
 // form wherever the launch still has a workgroup for every CU.
