@@ -135,22 +135,36 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepPair pair) {
     }
 
     f32x4 st[KT];
-#pragma unroll
-    for (int kt = 0; kt < KT; ++kt) st[kt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-
     const int64_t nblk = (n + 63) / 64;
     // Sequence chunking (chunk-parallel variant): this workgroup produces the blocks
-    // [it_first, it_end) of the walk.  It first runs over the blocks before it_first with the
-    // state update only ("warm-up": y and z are read, nothing is written) to rebuild the state
-    // its chunk starts from; there is no hand-off between workgroups and no workspace.
-    const int64_t it_first = a.chunk_start[chunk];
-    const int64_t it_end = a.chunk_start[chunk + 1];
-    // Two register sets of prefetched tiles (feature dims up to 128; wider ones have no registers
-    // to spare and keep one): while block `it` is worked on, block it+1 sits in LDS and blocks
-    // it+2, it+3 are in flight from memory (one block of prefetch does not cover the memory
-    // latency under load).
-    constexpr int NSET = DKP <= 128 ? 2 : 1;
-    u32x4 xrA[XC], yrA[XC], zrA, xrB[XC], yrB[XC], zrB;
+    // [it_first, it_end) of the walk.  Without a workspace (kWarmUp) it first runs over the blocks
+    // before it_first with the state update only ("warm-up": y and z are read, nothing is written)
+    // to rebuild the state its chunk starts from.  With one, the chunks are equally long and a
+    // workgroup walks its own chunk only: first with the state update alone, from zero, to leave the
+    // state it ends with (kCollect), then - a scan kernel having combined those into the state at the
+    // start of every chunk - for good, from that state (kApply).
+    const int mode = pair.mode;
+    const int nchunk = pair.a[0].nchunk;
+    if (mode == kCollect && chunk == nchunk - 1) return;  // nobody needs the state after the last chunk
+    const int64_t cbeg = mode == kWarmUp ? (int64_t)a.chunk_start[chunk] : min((int64_t)chunk * pair.chunk_len, nblk);
+    const int64_t cend = mode == kWarmUp ? (int64_t)a.chunk_start[chunk + 1] : min((int64_t)(chunk + 1) * pair.chunk_len, nblk);
+    const int64_t it0 = mode == kWarmUp ? 0 : cbeg;           // first block this workgroup walks
+    const int64_t it_first = mode == kCollect ? cend : cbeg;  // first block whose output it produces
+    const int64_t it_end = cend;
+    // state slots: [unit][sweep][slice][chunk 0 .. nchunk-2][state wave][tile][lane] accumulator quartets
+    constexpr size_t SF = (size_t)4 * KT * 64 * 4;
+    float* const slot0 = pair.state + ((((size_t)unit * nprod + sub % nprod) * nslice + slice) * (size_t)(nchunk - 1)) * SF;
+    const size_t lane_slot = ((size_t)w * KT * 64 + lane) * 4;
+    {
+        const bool resume = mode == kApply && chunk > 0 && state_role;
+        const float* const src = slot0 + (size_t)(chunk - 1) * SF + lane_slot;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+            st[kt] = resume ? *reinterpret_cast<const f32x4*>(src + (size_t)kt * 256) : (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
+    // One register set of prefetched tiles (there are no registers to spare for two at these feature
+    // dims): while block `it` is worked on, block it+1 is in flight from memory.
+    u32x4 xrA[XC], yrA[XC], zrA;
 
     // Per-lane byte offsets of this thread's 16-byte chunks inside a 64-token block (out of range
     // where the chunk lies in the zero padding dk..DKP-1 or beyond dv); the block's first token goes
@@ -214,10 +228,9 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepPair pair) {
 
     // zero P once: tiles on the masked side of the diagonal are never written
     for (int c = tid; c < 64 * ZS / 8; c += 512) reinterpret_cast<uint4*>(Ps)[c] = make_uint4(0, 0, 0, 0);
-    load_block(0, xrA, yrA, zrA);
-    if (NSET == 2) load_block(1, xrB, yrB, zrB);
-    stage_block(0, xrA, yrA, zrA);
-    load_block(NSET == 2 ? 2 : 1, xrA, yrA, zrA);
+    load_block(it0, xrA, yrA, zrA);
+    stage_block(NBUF == 2 ? (int)(it0 & 1) : 0, xrA, yrA, zrA);
+    load_block(it0 + 1, xrA, yrA, zrA);
     __syncthreads();
 
     // One block of the walk.  `xr, yr, zr` hold block it+1 on entry and block it+3 on exit.
@@ -229,13 +242,6 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepPair pair) {
         const T* Xs = tiles + buf * L::TILE;
         const T* Ys = Xs + 64 * XS;
         const T* Zs = Ys + 64 * XS;
-        if (NSET == 2) {
-            // publish block it+1 (its LDS buffer was last read in block it-1) and refill the
-            // registers with block it+3: both overlap the matrix work below
-            stage_block((int)((it + 1) & 1), xr, yr, zr);
-            load_block(it + 3, xr, yr, zr);
-        }
-
         // =================== phase 1 =========================================
         if (warm) {
             // nothing: x is not needed and no output is produced
@@ -397,7 +403,7 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepPair pair) {
                     buf_store8(ob, off, tok < nrows ? tok * ots * (unsigned)sizeof(T) : 0u, __builtin_bit_cast(u32x2, o));
                 }
             }
-        } else if (cols_active && have_next) {
+        } else if (cols_active && (have_next || mode == kCollect)) {
             // state = lam^64 state + y^T (z * Lupd)
             V8 zf[2];
 #pragma unroll
@@ -436,9 +442,7 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepPair pair) {
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        if (NSET == 2) {
-            __syncthreads();
-        } else if (NBUF == 2) {
+        if (NBUF == 2) {
             stage_block((int)((it + 1) & 1), xr, yr, zr);
             load_block(it + 2, xr, yr, zr);
             __syncthreads();
@@ -449,23 +453,18 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepPair pair) {
             __syncthreads();
         }
     };
-    if (NSET == 2) {
-        // Both halves of the unrolled loop always run, so the two register sets are refilled in the
-        // same order on every path and the wait before staging one set leaves the other in flight.
-        int64_t it = 0;
-        for (; it + 1 < it_end; it += 2) {
-            block_body(it, xrB, yrB, zrB);
-            block_body(it + 1, xrA, yrA, zrA);
-        }
-        if (it < it_end) block_body(it, xrB, yrB, zrB);
-    } else {
-        for (int64_t it = 0; it < it_end; ++it) block_body(it, xrA, yrA, zrA);
+    for (int64_t it = it0; it < it_end; ++it) block_body(it, xrA, yrA, zrA);
+    if (mode == kCollect && state_role) {
+        float* const dst = slot0 + (size_t)chunk * SF + lane_slot;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<f32x4*>(dst + (size_t)kt * 256) = st[kt];
     }
 }
 
 template <typename T, int DKP, bool REVERSE, bool DECAY>
 static int launch_one(const SweepPair& pair, hipStream_t st) {
     const SweepArgs& a = pair.a[0];
+    if (pair.mode != kWarmUp && pipe_state_floats(a.dk, false) != (size_t)4 * (DKP / 16) * 64 * 4) return LA_E_WORKSPACE;
     constexpr size_t lds = SweepLds<DKP>::bytes(sizeof(T));
     static_assert(lds <= 160 * 1024, "LDS budget");
     auto kern = la_sweep_kernel<T, DKP, REVERSE, DECAY>;
@@ -570,14 +569,31 @@ static SweepArgs make_args(const SweepIO& io, const float* s, int64_t bh, int64_
     return a;
 }
 
-static int launch_classic(const SweepPair& p, int dtype, bool reverse, hipStream_t st) {
+static int launch_classic_one(const SweepPair& p, int dtype, bool reverse, hipStream_t st) {
     if (dtype == LA_BF16) return reverse ? launch_dir<__bf16, true>(p, st) : launch_dir<__bf16, false>(p, st);
     if (dtype == LA_FP16) return reverse ? launch_dir<_Float16, true>(p, st) : launch_dir<_Float16, false>(p, st);
     return LA_E_UNSUPPORTED;
 }
 
-// With a workspace the pipelined kernel does not rebuild a chunk's incoming state with warm-up blocks:
-// it collects the states the chunks end with, scans them and starts every chunk from the result (three
+// The two-barrier kernel (feature dims 129..256), in one launch or - chunks with scanned states - three.
+static int launch_classic(const SweepPair& p, int dtype, bool reverse, hipStream_t st) {
+    SweepPair q = p;
+    if (p.mode == kWarmUp || p.a[0].nchunk <= 1) {
+        q.mode = kWarmUp;
+        return launch_classic_one(q, dtype, reverse, st);
+    }
+    if (!p.state || p.chunk_len < 1) return LA_E_WORKSPACE;
+    q.mode = kCollect;
+    int rc = launch_classic_one(q, dtype, reverse, st);
+    if (rc != LA_OK) return rc;
+    rc = launch_state_scan(p, st);
+    if (rc != LA_OK) return rc;
+    q.mode = kApply;
+    return launch_classic_one(q, dtype, reverse, st);
+}
+
+// With a workspace the kernels do not rebuild a chunk's incoming state with warm-up blocks: the states
+// the chunks end with are collected and scanned, and every chunk starts from the result (three
 // launches; equally long chunks, up to 64 of them).  Number of chunks and bytes of workspace for a
 // launch of nprod sweeps, 0 bytes where the warm-up form is used.  LA_SWEEP_SCAN=0 keeps to the warm-up form.
 struct ScanPlan {
@@ -587,7 +603,7 @@ struct ScanPlan {
 static ScanPlan plan_scan(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, bool wide) {
     ScanPlan pl = {1, 0, 0};
     const char* off = getenv("LA_SWEEP_SCAN");
-    if (dk > 128 || (off && atoi(off) == 0)) return pl;
+    if (off && atoi(off) == 0) return pl;
     const char* env = getenv("LA_SWEEP_CHUNKS");
     const int forced = env ? atoi(env) : 0;
     const int64_t nblk = (n + 63) / 64, cus = num_cus();
@@ -609,7 +625,7 @@ static ScanPlan plan_scan(int64_t bh, int64_t n, int64_t dk, int64_t dv, int npr
     return pl;
 }
 
-// Workspace the pipelined kernel can use for one launch of nprod sweeps (0: none).
+// Workspace the kernels can use for one launch of nprod sweeps (0: none).
 size_t sweep_workspace_bytes(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int dtype) {
     if (dtype != LA_BF16 && dtype != LA_FP16) return 0;
     return plan_scan(bh, n, dk, dv, nprod, wide_columns(bh, n, dk, dv, nprod)).bytes;

@@ -116,9 +116,14 @@ struct SweepPair {
 // n, dk, dv, h, bh, nslice and the chunking must agree between the two sweeps of a pair.
 enum { kWarmUp = 0, kCollect = 1, kApply = 2 };
 int sweep_pipe(const SweepPair& p, int dtype, bool reverse, hipStream_t st);
-// Floats of one state slot of the pipelined kernel (dk padded to 64 or 128, 64 or 128 columns): must
-// agree with the kernel's own SF.
-// (the 128-column form exists for the 128-wide feature tile only)
-inline size_t pipe_state_floats(int dk, bool wide) { return (size_t)(dk <= 64 && !wide ? 64 : 128) * (wide ? 128 : 64); }
+// Floats of one state slot: the feature dim as the kernel pads it (64 or 128 in the pipelined kernel, 192
+// or 256 in the two-barrier one) times the 64 or 128 columns of a workgroup.  Must agree with the
+// kernels' own SF; the 128-column form exists for the 128-wide feature tile only.
+inline size_t pipe_state_floats(int dk, bool wide) {
+    const int dkp = dk > 192 ? 256 : dk > 128 ? 192 : (dk <= 64 && !wide ? 64 : 128);
+    return (size_t)dkp * (wide ? 128 : 64);
+}
+// Between a kCollect and a kApply launch: scans the chunks' end states in place (la_sweep_pipe.hip).
+int launch_state_scan(const SweepPair& p, hipStream_t st);
 
 }  // namespace la

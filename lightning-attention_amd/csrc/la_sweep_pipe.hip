@@ -657,6 +657,16 @@ __global__ __launch_bounds__(256) void la_state_scan_kernel(float* state, const 
     }
 }
 
+int launch_state_scan(const SweepPair& p, hipStream_t st) {
+    const SweepArgs& a = p.a[0];
+    const int quartets = (int)(pipe_state_floats(a.dk, p.wide != 0) / 4);
+    const int sets_per_unit = p.nprod * a.nslice;
+    const int64_t nblk = (a.n + 63) / 64;
+    hipLaunchKernelGGL(la_state_scan_kernel, dim3((unsigned)((quartets + 255) / 256), (unsigned)(a.bh * sets_per_unit)),
+                       dim3(256), 0, st, p.state, a.s, a.h, sets_per_unit, a.nchunk, p.chunk_len, nblk, quartets);
+    return (int)hipGetLastError();
+}
+
 static int launch_any(const SweepPair& p, int dtype, bool reverse, hipStream_t st) {
     if (dtype == LA_BF16) return reverse ? launch_dir<__bf16, true>(p, st) : launch_dir<__bf16, false>(p, st);
     if (dtype == LA_FP16) return reverse ? launch_dir<_Float16, true>(p, st) : launch_dir<_Float16, false>(p, st);
@@ -677,12 +687,7 @@ int sweep_pipe(const SweepPair& p, int dtype, bool reverse, hipStream_t st) {
     q.mode = kCollect;
     int rc = launch_any(q, dtype, reverse, st);
     if (rc != LA_OK) return rc;
-    const int quartets = (int)(pipe_state_floats(a.dk, p.wide != 0) / 4);
-    const int sets_per_unit = p.nprod * a.nslice;
-    const int64_t nblk = (a.n + 63) / 64;
-    hipLaunchKernelGGL(la_state_scan_kernel, dim3((unsigned)((quartets + 255) / 256), (unsigned)(a.bh * sets_per_unit)),
-                       dim3(256), 0, st, p.state, a.s, a.h, sets_per_unit, a.nchunk, p.chunk_len, nblk, quartets);
-    rc = (int)hipGetLastError();
+    rc = launch_state_scan(p, st);
     if (rc != LA_OK) return rc;
     q.mode = kApply;
     return launch_any(q, dtype, reverse, st);

@@ -250,10 +250,11 @@ def test_sequence_chunking_is_exact(b, h, n, d, e, monkeypatch):
 
 
 @pytest.mark.parametrize("b, h, n, d, e", [(1, 2, 4096, 128, 64), (2, 3, 1000, 64, 128), (1, 2, 2100, 128, 128), (1, 1, 1500, 96, 72),
-                                           (3, 1, 831, 16, 128), (1, 2, 900, 64, 64)])
+                                           (3, 1, 831, 16, 128), (1, 2, 900, 64, 64), (1, 2, 1500, 192, 192), (1, 1, 900, 256, 256),
+                                           (2, 1, 1100, 160, 136)])
 @pytest.mark.parametrize("decay", [True, False])
 def test_chunk_states_by_scan(b, h, n, d, e, decay, monkeypatch):
-    """With a workspace (the Python operators always pass one) the d <= 128 kernel starts every chunk from
+    """With a workspace (the Python operators always pass one) the kernels start every chunk from
     a scanned state instead of rebuilding it: three launches, up to 64 chunks.  The state sums are taken
     in another order, so results agree with the single walk to rounding, not bit for bit."""
     q, k, v, do = make_inputs(b, h, n, d, e, torch.bfloat16, 1.0, seed=n + d)
