@@ -233,7 +233,7 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepPair pair) {
     load_block(it0 + 1, xrA, yrA, zrA);
     __syncthreads();
 
-    // One block of the walk.  `xr, yr, zr` hold block it+1 on entry and block it+3 on exit.
+    // One block of the walk.  `xr, yr, zr` hold block it+1 on entry and block it+2 on exit.
     auto block_body = [&](const int64_t it, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4& zr) {
         const int64_t t = REVERSE ? nblk - 1 - it : it;
         const bool have_next = it + 1 < it_end;
@@ -503,18 +503,22 @@ static int num_cus() {
 // rebuild their incoming state themselves.  A warm-up block costs about half a full block, so
 // chunk lengths shrink geometrically (len_c ~ (1 - rho)^c, rho = 0.5) to make all workgroups
 // finish together.  LA_SWEEP_CHUNKS=<C> overrides the count.
-static void choose_chunks(SweepArgs& a, int nprod = 1) {
-    const char* env = getenv("LA_SWEEP_CHUNKS");  // read per call so that tests can vary it
-    const int forced = env ? atoi(env) : 0;
-    const int cus = num_cus();
-    const int64_t nblk = (a.n + 63) / 64;
-    const int64_t wgs = (int64_t)((a.bh + 7) / 8 * 8) * a.nslice * nprod;
+static int64_t warm_up_chunks(int64_t wgs, int64_t nblk) {
+    const int64_t cus = num_cus();
     int64_t c = 1;
-    if (forced > 0) c = forced;
-    else if (wgs * 2 <= cus && nblk >= 8) {
+    if (wgs * 2 <= cus && nblk >= 8) {
         c = cus / wgs;
         if (c > nblk / 4) c = nblk / 4;
     }
+    return c > 8 ? 8 : c < 1 ? 1 : c;
+}
+
+static void choose_chunks(SweepArgs& a, int nprod = 1) {
+    const char* env = getenv("LA_SWEEP_CHUNKS");  // read per call so that tests can vary it
+    const int forced = env ? atoi(env) : 0;
+    const int64_t nblk = (a.n + 63) / 64;
+    const int64_t wgs = (int64_t)((a.bh + 7) / 8 * 8) * a.nslice * nprod;
+    int64_t c = forced > 0 ? forced : warm_up_chunks(wgs, nblk);
     if (c > 8) c = 8;
     if (c > nblk) c = nblk;
     if (c < 1) c = 1;
@@ -536,28 +540,6 @@ static void choose_chunks(SweepArgs& a, int nprod = 1) {
     a.nchunk = (int)c;
     a.chunk_start[c] = (int)nblk;
     for (int i = (int)c + 1; i < 9; ++i) a.chunk_start[i] = (int)nblk;
-}
-
-// The pipelined kernel can give each workgroup 128 columns of z / out instead of 64: the score tile
-// and the x / y tiles are then produced once per 128 output columns, and the power-limited kernel
-// turns the saved work into time (dK + dV at the headline shape: 0.31 against 0.415 ms) - as long
-// as there are workgroups enough.  A 128-column workgroup takes about 1.25 times as long as a
-// 64-column one, and there are half as many: compare the rounds of workgroups the chip has to run.
-// LA_SWEEP_WIDE=0 / 1 overrides the choice.
-static bool wide_columns(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod) {
-    if (dk > 128 || dv <= 64 || dv > 128) return false;
-    const char* env = getenv("LA_SWEEP_WIDE");
-    if (env) return atoi(env) != 0;
-    if (dk <= 64) return false;  // the 128-column form pads the feature dim to 128
-    const int64_t cus = num_cus(), wide = (bh + 7) / 8 * 8 * nprod, narrow = 2 * wide;
-    if (narrow <= cus) {
-        // Every 64-column workgroup gets a CU of its own.  With so few of them that a long walk is cut
-        // into chunks anyway, rather half as many workgroups of 128 columns and twice the chunks
-        // (b1 h32 n8192 fwd+bwd 0.28 against 0.34 ms, b1 h4 n65536 0.46 against 0.62).
-        const char* off = getenv("LA_SWEEP_SCAN");
-        return narrow * 2 <= cus && (n + 63) / 64 >= 128 && !(off && atoi(off) == 0);
-    }
-    return (wide + cus - 1) / cus * 5 < (narrow + cus - 1) / cus * 4;
 }
 
 static SweepArgs make_args(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv) {
@@ -599,11 +581,26 @@ static int launch_classic(const SweepPair& p, int dtype, bool reverse, hipStream
 struct ScanPlan {
     int nchunk, chunk_len;
     size_t bytes;
+    double us;  // estimated duration of the launch(es)
 };
+
+// Estimates, in microseconds, behind the choices below.  A workgroup takes about block_us per 64-token
+// block (measured, by feature dim and columns per workgroup) and half of that for a block it only folds
+// into the state.  Warm-up blocks: with the geometric chunk lengths of choose_chunks the longest
+// workgroup runs the fraction `frac` of a single walk.  Scanned states: a chunk one and a half times,
+// plus two more launches and the scan (16 us measured, and 10 for the host's share).
+static double block_us(int64_t dk, bool wide) { return dk <= 64 ? 1.0 : dk <= 128 ? (wide ? 1.75 : 1.4) : dk <= 192 ? 2.1 : 2.9; }
+static double warm_up_us(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, bool wide) {
+    static const double frac[9] = {1.0, 1.0, 0.77, 0.71, 0.68, 0.67, 0.66, 0.66, 0.66};
+    const int64_t nblk = (n + 63) / 64, wgs = (bh + 7) / 8 * 8 * (wide ? 1 : (dv + 63) / 64) * nprod;
+    return frac[warm_up_chunks(wgs, nblk)] * (double)nblk * block_us(dk, wide);
+}
+
 static ScanPlan plan_scan(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, bool wide) {
-    ScanPlan pl = {1, 0, 0};
+    const ScanPlan none = {1, 0, 0, warm_up_us(bh, n, dk, dv, nprod, wide)};
+    ScanPlan pl = none;
     const char* off = getenv("LA_SWEEP_SCAN");
-    if (off && atoi(off) == 0) return pl;
+    if (off && atoi(off) == 0) return none;
     const char* env = getenv("LA_SWEEP_CHUNKS");
     const int forced = env ? atoi(env) : 0;
     const int64_t nblk = (n + 63) / 64, cus = num_cus();
@@ -611,36 +608,62 @@ static ScanPlan plan_scan(int64_t bh, int64_t n, int64_t dk, int64_t dv, int npr
     const int64_t wgs = (bh + 7) / 8 * 8 * nslice * nprod;
     int64_t c = 1;
     if (forced > 0) c = forced;
-    else if (wgs * 2 <= cus && nblk >= 128) {  // (shorter walks: three launches cost more than warm-up blocks)
+    else if (wgs * 2 <= cus) {
         c = cus / wgs;
         if (c > nblk / 4) c = nblk / 4;  // at least four blocks per chunk
     }
     if (c > 64) c = 64;
     if (c > nblk) c = nblk;
-    if (c < 2) return pl;
+    if (c < 2) return none;
     pl.chunk_len = (int)((nblk + c - 1) / c);
+    pl.us = 1.5 * pl.chunk_len * block_us(dk, wide) + 16.0 + 10.0;
+    if (forced <= 0 && pl.us >= none.us) return none;
     pl.nchunk = (int)((nblk + pl.chunk_len - 1) / pl.chunk_len);  // no empty chunk
-    if (pl.nchunk < 2 || bh * nprod * nslice > 65535) return ScanPlan{1, 0, 0};
+    if (pl.nchunk < 2 || bh * nprod * nslice > 65535) return none;
     pl.bytes = (size_t)(bh * nprod * nslice) * (size_t)(pl.nchunk - 1) * pipe_state_floats((int)dk, wide) * sizeof(float);
     return pl;
+}
+
+// The pipelined kernel can give each workgroup 128 columns of z / out instead of 64: the score tile
+// and the x / y tiles are then produced once per 128 output columns, and the power-limited kernel
+// turns the saved work into time (dK + dV at the headline shape: 0.31 against 0.415 ms) - as long
+// as there are workgroups enough.  A 128-column workgroup takes about 1.25 times as long as a
+// 64-column one, and there are half as many: compare the rounds of workgroups the chip has to run.
+// `scratch`: bytes of workspace the caller has.  LA_SWEEP_WIDE=0 / 1 overrides the choice.
+static bool wide_columns(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, size_t scratch) {
+    if (dk > 128 || dv <= 64 || dv > 128) return false;
+    const char* env = getenv("LA_SWEEP_WIDE");
+    if (env) return atoi(env) != 0;
+    if (dk <= 64) return false;  // the 128-column form pads the feature dim to 128
+    const int64_t cus = num_cus(), wide = (bh + 7) / 8 * 8 * nprod, narrow = 2 * wide;
+    if (narrow <= cus) {
+        // Every 64-column workgroup gets a CU of its own.  With so few of them that a long walk is cut
+        // into chunks from scanned states, rather half as many workgroups of 128 columns and twice the chunks
+        // (b1 h32 n8192 fwd+bwd 0.28 against 0.34 ms, b1 h4 n65536 0.46 against 0.62).
+        if (narrow * 2 > cus) return false;
+        const ScanPlan w = plan_scan(bh, n, dk, dv, nprod, true), nw = plan_scan(bh, n, dk, dv, nprod, false);
+        return w.nchunk > 1 && w.bytes <= scratch && w.us < (nw.bytes <= scratch ? nw.us : warm_up_us(bh, n, dk, dv, nprod, false));
+    }
+    return (wide + cus - 1) / cus * 5 < (narrow + cus - 1) / cus * 4;
 }
 
 // Workspace the kernels can use for one launch of nprod sweeps (0: none).
 size_t sweep_workspace_bytes(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int dtype) {
     if (dtype != LA_BF16 && dtype != LA_FP16) return 0;
-    return plan_scan(bh, n, dk, dv, nprod, wide_columns(bh, n, dk, dv, nprod)).bytes;
+    return plan_scan(bh, n, dk, dv, nprod, wide_columns(bh, n, dk, dv, nprod, (size_t)-1)).bytes;
 }
 
 static int launch_planned(SweepPair& p, int64_t bh, int64_t n, int64_t dk, int64_t dv, int dtype, bool reverse, void* ws,
                           size_t ws_bytes, hipStream_t st) {
-    p.wide = wide_columns(bh, n, dk, dv, p.nprod) ? 1 : 0;
+    const bool ws_ok = ws && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0;
+    p.wide = wide_columns(bh, n, dk, dv, p.nprod, ws_ok ? ws_bytes : 0) ? 1 : 0;
     p.mode = kWarmUp;
     p.chunk_len = 0;
     p.state = nullptr;
     for (int i = 0; i < p.nprod; ++i)
         if (p.wide) p.a[i].nslice = 1;
     const ScanPlan pl = plan_scan(bh, n, dk, dv, p.nprod, p.wide != 0);
-    if (pl.nchunk > 1 && ws && ws_bytes >= pl.bytes && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0) {
+    if (pl.nchunk > 1 && ws_ok && ws_bytes >= pl.bytes) {
         p.mode = kCollect;  // sweep_pipe runs the three launches
         p.chunk_len = pl.chunk_len;
         p.state = static_cast<float*>(ws);

@@ -37,12 +37,14 @@ def test_host_only_entry_points():
         assert L.la_supported(d, e, dt) == want, (d, e, dt)
     assert L.la_error_string(0) == b"success"
     assert b"NULL" in L.la_error_string(-1)
-    # scratch for the chunked walk: none when the sequences fill the chip, short walks, wide dims or float32;
+    # scratch for the chunked walk: none when the sequences fill the chip, for short walks or float32;
     # otherwise one d x e (padded) float state per chunk but the last, per sequence and column slice
     assert L.la_workspace_bytes(0, 4, 32, 8192, 128, 128, 0) == 0
     assert L.la_workspace_bytes(1, 4, 32, 8192, 128, 128, 0) == 0
     assert L.la_workspace_bytes(0, 1, 8, 2048, 128, 128, 0) == 0
-    assert L.la_workspace_bytes(0, 1, 8, 8192, 192, 192, 0) == 0
+    assert L.la_workspace_bytes(0, 2, 12, 2048, 192, 192, 0) == 0
+    wide_dims = L.la_workspace_bytes(0, 1, 8, 8192, 192, 192, 0)
+    assert wide_dims > 0 and wide_dims % (8 * 3 * 192 * 64 * 4) == 0
     assert L.la_workspace_bytes(0, 1, 8, 8192, 128, 128, 2) == 0
     need = L.la_workspace_bytes(0, 1, 8, 8192, 128, 128, 0)
     assert need > 0 and need % (128 * 64 * 4) == 0 and need <= 8 * 2 * 63 * 128 * 64 * 4
