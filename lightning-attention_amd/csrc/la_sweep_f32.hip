@@ -4,10 +4,22 @@
 // row/column = lane % 16, contraction slot = lane / 16).  Nothing is rounded
 // below float32, so the result is within float32 accumulation error of the
 // exact value.  This is the accuracy path, not the throughput path.
+//
+// Every operand but z comes out of LDS in 16-byte reads.  A contraction may visit its index in any
+// order as long as both operands agree, and the rows of a state tile may stand for any 16 features
+// as long as the products that write and read the state agree:
+//   scores        step (kt, v) of slot g contracts feature 16kt + 4g + v: x and y rows read 4 floats at a time;
+//   state tiles   come in groups of four (kt = 4K + q); row rho of tile kt is feature
+//                 64K + 4 pi(rho) + q with pi(rho) = 4 (rho % 4) + rho / 4, so that one 16-byte read of a
+//                 y row (state update) or an x row (inter-block term) feeds the four tiles of a group.
 #include "la_common.h"
 #include "lightning_attn_hip.h"
 
 namespace la {
+
+#ifndef LA_F32_XPAD
+#define LA_F32_XPAD 8  // floats of padding per x / y row
+#endif
 
 struct SweepArgsF32 {
     const float* x;
@@ -25,9 +37,10 @@ __device__ __forceinline__ f32x4 mma4(float a, float b, f32x4 c) {
 
 template <int DKP, bool REVERSE, bool DECAY>
 __global__ __launch_bounds__(256, 1) void la_sweep_f32_kernel(SweepArgsF32 a) {
-    constexpr int XS = DKP + 4;   // row stride (floats) of the x / y tiles
+    constexpr int XS = DKP + LA_F32_XPAD;  // row stride (floats) of the x / y tiles
     constexpr int ZS = 64 + 4;    // row stride of the z slice and the P tile
     constexpr int KT = DKP / 16;  // 16-row state tiles
+    constexpr int KG = DKP / 64;  // groups of four state tiles
     constexpr int XC = DKP / 16;  // 16-byte chunks per thread for an x / y tile
     extern __shared__ __align__(16) unsigned char smem[];
     float* Xs = reinterpret_cast<float*>(smem);
@@ -130,12 +143,16 @@ __global__ __launch_bounds__(256, 1) void la_sweep_f32_kernel(SweepArgsF32 a) {
             f32x4 sacc[4];
 #pragma unroll
             for (int jt = 0; jt < 4; ++jt) sacc[jt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-            for (int k0 = 0; k0 < DKP; k0 += 4) {
-                const float bx = Xs[(16 * w + r) * XS + k0 + g];
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+                const f32x4 bx = *reinterpret_cast<const f32x4*>(Xs + (16 * w + r) * XS + 16 * kt + 4 * g);
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) {
-                    if (jt >= jlo && jt <= jhi) sacc[jt] = mma4(Ys[(16 * jt + r) * XS + k0 + g], bx, sacc[jt]);
+                    if (jt >= jlo && jt <= jhi) {
+                        const f32x4 ay = *reinterpret_cast<const f32x4*>(Ys + (16 * jt + r) * XS + 16 * kt + 4 * g);
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) sacc[jt] = mma4(ay[v], bx[v], sacc[jt]);
+                    }
                 }
             }
 #pragma unroll
@@ -162,12 +179,15 @@ __global__ __launch_bounds__(256, 1) void la_sweep_f32_kernel(SweepArgsF32 a) {
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
                 oacc[i4] = (f32x4){0.f, 0.f, 0.f, 0.f};
-                // 2a. inter-block: contraction slot g of step (kt, v) is feature 16kt + 4g + v
+                // 2a. inter-block: st[4K + q][v] holds row 4g + v of its tile, feature 64K + 16v + 4g + q
 #pragma unroll
-                for (int kt = 0; kt < KT; ++kt) {
-                    const f32x4 bx = *reinterpret_cast<const f32x4*>(Xs + (16 * i4 + r) * XS + 16 * kt + 4 * g);
+                for (int K = 0; K < KG; ++K) {
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) oacc[i4] = mma4(st[kt][v], bx[v], oacc[i4]);
+                    for (int v = 0; v < 4; ++v) {
+                        const f32x4 bx = *reinterpret_cast<const f32x4*>(Xs + (16 * i4 + r) * XS + 64 * K + 16 * v + 4 * g);
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) oacc[i4] = mma4(st[4 * K + q][v], bx[q], oacc[i4]);
+                    }
                 }
                 if (DECAY) {
 #pragma unroll
@@ -202,13 +222,18 @@ __global__ __launch_bounds__(256, 1) void la_sweep_f32_kernel(SweepArgsF32 a) {
 #pragma unroll
                         for (int v = 0; v < 4; ++v) st[kt][v] *= lamB;
                 }
+                // row r of tile 4K + q is feature 64K + 16 (r % 4) + 4 (r / 4) + q
 #pragma unroll
-                for (int kt = 0; kt < KT; ++kt) {
+                for (int K = 0; K < KG; ++K) {
 #pragma unroll
                     for (int jt = 0; jt < 4; ++jt)
 #pragma unroll
-                        for (int v = 0; v < 4; ++v)
-                            st[kt] = mma4(Ys[(16 * jt + 4 * g + v) * XS + 16 * kt + r], zf[jt][v], st[kt]);
+                        for (int v = 0; v < 4; ++v) {
+                            const f32x4 ay = *reinterpret_cast<const f32x4*>(Ys + (16 * jt + 4 * g + v) * XS + 64 * K +
+                                                                             16 * (r & 3) + 4 * (r >> 2));
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) st[4 * K + q] = mma4(ay[q], zf[jt][v], st[4 * K + q]);
+                        }
                 }
             }
         }
@@ -222,7 +247,7 @@ __global__ __launch_bounds__(256, 1) void la_sweep_f32_kernel(SweepArgsF32 a) {
 
 template <int DKP, bool REVERSE, bool DECAY>
 static int launch_one_f32(const SweepArgsF32& a, hipStream_t st) {
-    constexpr size_t lds = (size_t)(2 * 64 * (DKP + 4) + 2 * 64 * 68) * sizeof(float);
+    constexpr size_t lds = (size_t)(2 * 64 * (DKP + LA_F32_XPAD) + 2 * 64 * 68) * sizeof(float);
     auto kern = la_sweep_f32_kernel<DKP, REVERSE, DECAY>;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -238,7 +263,6 @@ template <bool REVERSE>
 static int launch_dir_f32(const SweepArgsF32& a, hipStream_t st) {
     const bool decay = a.s != nullptr;
 #define LA_GO(DKP) (decay ? launch_one_f32<DKP, REVERSE, true>(a, st) : launch_one_f32<DKP, REVERSE, false>(a, st))
-    if (a.dk <= 32) return LA_GO(32);
     if (a.dk <= 64) return LA_GO(64);
     return LA_GO(128);
 #undef LA_GO
