@@ -7,6 +7,8 @@
 namespace la {
 int sweep(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
           bool reverse, void* ws, size_t ws_bytes, hipStream_t st);
+int sweep_bwd_once(const SweepIO& dq, const SweepIO& dk, const SweepIO& dv, const float* s, int64_t bh, int64_t h, int64_t n,
+                   int64_t d, int dtype, void* ws, size_t ws_bytes, hipStream_t st);
 int sweep2(const SweepIO& io0, const SweepIO& io1, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv,
            int dtype, bool reverse, void* ws, size_t ws_bytes, hipStream_t st);
 size_t sweep_workspace_bytes(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int dtype);
@@ -98,6 +100,12 @@ static int bwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s
         if ((rc = check_tensor(*ts[i], b, h, n, cols[i], dtype)) != LA_OK) return rc;
     // dQ_i = sum_{j<=i} lam^(i-j) (dO_i . v_j) k_j
     // (the launches follow each other on one stream, so they can all use the same scratch memory)
+    if (d == e && dtype != LA_FP32) {
+        // few sequences: all three gradients in one launch, side by side (LA_E_UNSUPPORTED: not this time)
+        rc = sweep_bwd_once(io(dout, v, k, dq), io(v, dout, q, dk), io(k, q, dout, dv), s, b * h, h, n, d, dtype, ws.p,
+                            ws.bytes, st);
+        if (rc != LA_E_UNSUPPORTED) return rc;
+    }
     rc = run(dout, v, k, dq, s, b * h, h, n, e, d, dtype, false, ws, st);
     if (rc != LA_OK) return rc;
     // dK_j = sum_{i>=j} lam^(i-j) (v_j . dO_i) q_i   and   dV_j = sum_{i>=j} lam^(i-j) (k_j . q_i) dO_i

@@ -45,8 +45,9 @@ struct SweepLds {
     static constexpr size_t bytes(size_t elt) { return (size_t)(NBUF * TILE + 64 * ZS) * elt + 4 * 4 * 64 * 16; }
 };
 
+// `bid`: number of the workgroup within its part of the launch.
 template <typename T, int DKP, bool REVERSE, bool DECAY>
-__global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepPair pair) {
+__device__ __forceinline__ void sweep_body(const SweepPair& pair, const unsigned bid) {
     typedef Mma<T> M;
     typedef typename M::V8 V8;
     typedef typename M::V4 V4;
@@ -62,7 +63,7 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepPair pair) {
 
     // Workgroups are dealt round-robin to the 8 XCDs by linear id; keep the
     // column slices of one head on one XCD so their x / y re-reads share an L2.
-    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int xcd = bid & 7, local = bid >> 3;
     const int nslice = pair.a[0].nslice, nprod = pair.nprod;
     const int per_unit = nslice * pair.a[0].nchunk * nprod;
     const int unit = xcd + 8 * (local / per_unit);
@@ -462,6 +463,44 @@ __global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepPair pair) {
 }
 
 template <typename T, int DKP, bool REVERSE, bool DECAY>
+__global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepPair pair) {
+    sweep_body<T, DKP, REVERSE, DECAY>(pair, blockIdx.x);
+}
+
+// Forward-walking and backward-walking sweeps in one launch (SweepBoth).
+template <typename T, int DKP, bool DECAY>
+__global__ __launch_bounds__(512, 1) void la_sweep_both_kernel(SweepBoth both) {
+    if (blockIdx.x < both.nfwd) sweep_body<T, DKP, false, DECAY>(both.fwd, blockIdx.x);
+    else sweep_body<T, DKP, true, DECAY>(both.rev, blockIdx.x - both.nfwd);
+}
+
+static unsigned part_grid(const SweepPair& p) {
+    return (unsigned)((p.a[0].bh + 7) / 8 * 8 * p.a[0].nslice * p.a[0].nchunk * p.nprod);
+}
+
+template <typename T, int DKP, bool DECAY>
+static int launch_both_one(const SweepBoth& b, hipStream_t st) {
+    constexpr size_t lds = SweepLds<DKP>::bytes(sizeof(T));
+    auto kern = la_sweep_both_kernel<T, DKP, DECAY>;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+    }
+    hipLaunchKernelGGL(kern, dim3(b.nfwd + part_grid(b.rev)), dim3(512), lds, st, b);
+    return (int)hipGetLastError();
+}
+
+template <typename T>
+static int launch_both(const SweepBoth& b, hipStream_t st) {
+    const bool decay = b.fwd.a[0].s != nullptr;
+#define LA_GO(DKP) (decay ? launch_both_one<T, DKP, true>(b, st) : launch_both_one<T, DKP, false>(b, st))
+    if (b.fwd.a[0].dk <= 192) return LA_GO(192);
+    return LA_GO(256);
+#undef LA_GO
+}
+
+template <typename T, int DKP, bool REVERSE, bool DECAY>
 static int launch_one(const SweepPair& pair, hipStream_t st) {
     const SweepArgs& a = pair.a[0];
     if (pair.mode != kWarmUp && pipe_state_floats(a.dk, false) != (size_t)4 * (DKP / 16) * 64 * 4) return LA_E_WORKSPACE;
@@ -590,10 +629,13 @@ struct ScanPlan {
 // workgroup runs the fraction `frac` of a single walk.  Scanned states: a chunk one and a half times,
 // plus two more launches and the scan (16 us measured, and 10 for the host's share).
 static double block_us(int64_t dk, bool wide) { return dk <= 64 ? 1.0 : dk <= 128 ? (wide ? 1.75 : 1.4) : dk <= 192 ? 2.1 : 2.9; }
-static double warm_up_us(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, bool wide) {
+static double warm_up_frac(int64_t wgs, int64_t nblk) {
     static const double frac[9] = {1.0, 1.0, 0.77, 0.71, 0.68, 0.67, 0.66, 0.66, 0.66};
+    return frac[warm_up_chunks(wgs, nblk)];
+}
+static double warm_up_us(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, bool wide) {
     const int64_t nblk = (n + 63) / 64, wgs = (bh + 7) / 8 * 8 * (wide ? 1 : (dv + 63) / 64) * nprod;
-    return frac[warm_up_chunks(wgs, nblk)] * (double)nblk * block_us(dk, wide);
+    return warm_up_frac(wgs, nblk) * (double)nblk * block_us(dk, wide);
 }
 
 static ScanPlan plan_scan(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, bool wide) {
@@ -704,6 +746,60 @@ int sweep2(const SweepIO& io0, const SweepIO& io1, const float* s, int64_t bh, i
     p.a[0] = make_args(io0, s, bh, h, n, dk, dv);
     p.a[1] = make_args(io1, s, bh, h, n, dk, dv);
     return launch_planned(p, bh, n, dk, dv, dtype, reverse, ws, ws_bytes, st);
+}
+
+// The three sweeps of a backward pass with d == e (dQ forward; dK, dV reverse, paired) in ONE launch,
+// where that is the faster way: they fit on the chip together, so they run side by side, each cut into
+// the warm-up chunks the CUs left over allow.  Results are bit-identical to separate launches.
+// Returns LA_E_UNSUPPORTED when separate launches are to be used (they are estimated faster - scanned
+// chunk states on a long walk -, or the sweeps fill the chip anyway).  LA_SWEEP_ONCE=0 / 1: never /
+// whenever possible.
+int sweep_bwd_once(const SweepIO& dq, const SweepIO& dk, const SweepIO& dv, const float* s, int64_t bh, int64_t h, int64_t n,
+                   int64_t d, int dtype, void* ws, size_t ws_bytes, hipStream_t st) {
+    if (dtype != LA_BF16 && dtype != LA_FP16) return LA_E_UNSUPPORTED;
+    const char* env = getenv("LA_SWEEP_ONCE");
+    const int forced = env ? (atoi(env) != 0 ? 1 : -1) : 0;
+    if (forced < 0 || getenv("LA_SWEEP_UNPAIRED")) return LA_E_UNSUPPORTED;
+    const char* wide_env = getenv("LA_SWEEP_WIDE");
+    if (forced == 0 && wide_env && atoi(wide_env) != 0) return LA_E_UNSUPPORTED;  // 128-column workgroups asked for
+    const int64_t cus = num_cus(), nblk = (n + 63) / 64, nslice = (d + 63) / 64;
+    const int64_t wgs = (bh + 7) / 8 * 8 * nslice * 3;  // one chunk each
+    if (forced == 0) {
+        if (wgs > cus) return LA_E_UNSUPPORTED;
+        // what the separate launches would take, by the estimates behind their own plans
+        const bool ws_ok = ws && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0;
+        double separate = 0.0;
+        for (int nprod = 1; nprod <= 2; ++nprod) {
+            const bool wide = wide_columns(bh, n, d, d, nprod, ws_ok ? ws_bytes : 0);
+            const ScanPlan pl = plan_scan(bh, n, d, d, nprod, wide);
+            separate += pl.nchunk > 1 && ws_ok && ws_bytes >= pl.bytes ? pl.us : warm_up_us(bh, n, d, d, nprod, wide);
+        }
+        // here: the longest workgroup of 3 * wgs/3 * c warm-up chunked ones
+        if (warm_up_frac(wgs, nblk) * (double)nblk * block_us(d, false) >= separate) return LA_E_UNSUPPORTED;
+    }
+    SweepBoth b;
+    b.fwd.nprod = 1;
+    b.fwd.a[0] = make_args(dq, s, bh, h, n, d, d);
+    b.rev.nprod = 2;
+    b.rev.a[0] = make_args(dk, s, bh, h, n, d, d);
+    b.rev.a[1] = make_args(dv, s, bh, h, n, d, d);
+    for (SweepPair* p : {&b.fwd, &b.rev}) {
+        p->wide = 0;
+        p->mode = kWarmUp;
+        p->chunk_len = 0;
+        p->state = nullptr;
+    }
+    // the same chunks for every sweep: what all of them together leave room for
+    choose_chunks(b.fwd.a[0], 3);
+    b.fwd.a[1] = b.fwd.a[0];
+    for (int i = 0; i < 2; ++i) {
+        b.rev.a[i].nchunk = b.fwd.a[0].nchunk;
+        for (int j = 0; j < 9; ++j) b.rev.a[i].chunk_start[j] = b.fwd.a[0].chunk_start[j];
+    }
+    b.nfwd = part_grid(b.fwd);
+    if (d <= 128) return sweep_pipe_both(b, dtype, st);
+    if (dtype == LA_BF16) return launch_both<__bf16>(b, st);
+    return launch_both<_Float16>(b, st);
 }
 
 }  // namespace la

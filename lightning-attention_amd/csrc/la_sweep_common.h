@@ -112,6 +112,16 @@ struct SweepPair {
     float* state;
 };
 
+// One launch can also carry sweeps of both directions: the whole backward pass when d == e, dQ walking
+// forward, dK and dV backward.  That pays when the three sweeps together leave CUs idle (few
+// sequences): they run side by side instead of one after the other.  Warm-up chunking only; both
+// parts use the same kernel instantiation (64 columns per workgroup).
+struct SweepBoth {
+    SweepPair fwd, rev;
+    unsigned nfwd;  // workgroups of the forward part (a multiple of 8); the reverse part follows
+};
+int sweep_pipe_both(const SweepBoth& b, int dtype, hipStream_t st);  // feature dim up to 128, la_sweep_pipe.hip
+
 // Launches the single-barrier pipelined kernel (feature dim up to 128); defined in la_sweep_pipe.hip.
 // n, dk, dv, h, bh, nslice and the chunking must agree between the two sweeps of a pair.
 enum { kWarmUp = 0, kCollect = 1, kApply = 2 };

@@ -57,8 +57,9 @@ struct PipeLds {
 
 // DENSE: all four tensors are plain (b, h, n, d) arrays; their rows then take a shorter addressing path
 // (see load_block).
+// `bid`: number of the workgroup within its part of the launch.
 template <typename T, int DKP, int NH, bool REVERSE, bool DECAY, bool DENSE>
-__global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
+__device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const unsigned bid) {
     typedef Mma<T> M;
     typedef typename M::V8 V8;
     typedef typename M::V4 V4;
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
 
     // Workgroups are dealt round-robin to the 8 XCDs by linear id; keep the
     // column slices of one head on one XCD so their x / y re-reads share an L2.
-    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int xcd = bid & 7, local = bid >> 3;
     const int nslice = pair.a[0].nslice, nprod = pair.nprod;
     const int per_unit = nslice * pair.a[0].nchunk * nprod;
     const int unit = xcd + 8 * (local / per_unit);
@@ -596,6 +597,18 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
 }
 
 template <typename T, int DKP, int NH, bool REVERSE, bool DECAY, bool DENSE>
+__global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
+    sweep_pipe_body<T, DKP, NH, REVERSE, DECAY, DENSE>(pair, blockIdx.x);
+}
+
+// Forward-walking and backward-walking sweeps in one launch (SweepBoth).
+template <typename T, int DKP, bool DECAY, bool DENSE>
+__global__ __launch_bounds__(512, 1) void la_sweep_pipe_both_kernel(SweepBoth both) {
+    if (blockIdx.x < both.nfwd) sweep_pipe_body<T, DKP, 1, false, DECAY, DENSE>(both.fwd, blockIdx.x);
+    else sweep_pipe_body<T, DKP, 1, true, DECAY, DENSE>(both.rev, blockIdx.x - both.nfwd);
+}
+
+template <typename T, int DKP, int NH, bool REVERSE, bool DECAY, bool DENSE>
 static int launch_one(const SweepPair& pair, hipStream_t st) {
     const SweepArgs& a = pair.a[0];
     constexpr size_t lds = PipeLds<DKP, NH>::bytes(sizeof(T));
@@ -635,6 +648,52 @@ static int launch_dir(const SweepPair& pair, hipStream_t st) {
     return LA_GO(128, 1);
 #undef LA_GO
 #undef LA_GO2
+}
+
+static unsigned part_grid(const SweepPair& p) {
+    return (unsigned)((p.a[0].bh + 7) / 8 * 8 * p.a[0].nslice * p.a[0].nchunk * p.nprod);
+}
+
+template <typename T, int DKP, bool DECAY, bool DENSE>
+static int launch_both_one(const SweepBoth& b, hipStream_t st) {
+    constexpr size_t lds = PipeLds<DKP, 1>::bytes(sizeof(T));
+    auto kern = la_sweep_pipe_both_kernel<T, DKP, DECAY, DENSE>;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+    }
+    hipLaunchKernelGGL(kern, dim3(b.nfwd + part_grid(b.rev)), dim3(512), lds, st, b);
+    return (int)hipGetLastError();
+}
+
+template <typename T>
+static int launch_both(const SweepBoth& b, hipStream_t st) {
+    const SweepArgs& a = b.fwd.a[0];
+    const bool decay = a.s != nullptr;
+    bool dense = true;
+    for (const SweepPair* p : {&b.fwd, &b.rev})
+        for (int i = 0; i < p->nprod; ++i) {
+            const SweepArgs& c = p->a[i];
+            dense = dense && plain(c.lx, c.h, c.n, c.dk) && plain(c.ly, c.h, c.n, c.dk) && plain(c.lz, c.h, c.n, c.dv) &&
+                    plain(c.lo, c.h, c.n, c.dv);
+        }
+#define LA_GO2(DKP, DENSE) (decay ? launch_both_one<T, DKP, true, DENSE>(b, st) : launch_both_one<T, DKP, false, DENSE>(b, st))
+#define LA_GO(DKP) (dense ? LA_GO2(DKP, true) : LA_GO2(DKP, false))
+    if (a.dk <= 64) return LA_GO(64);
+    return LA_GO(128);
+#undef LA_GO
+#undef LA_GO2
+}
+
+int sweep_pipe_both(const SweepBoth& b, int dtype, hipStream_t st) {
+    const SweepArgs &f = b.fwd.a[0], &r = b.rev.a[0];
+    if (f.dk > 128 || f.dk != r.dk || f.dv != r.dv || f.n != r.n || f.bh != r.bh || b.fwd.wide || b.rev.wide ||
+        b.fwd.mode != kWarmUp || b.rev.mode != kWarmUp || b.nfwd != part_grid(b.fwd))
+        return LA_E_UNSUPPORTED;
+    if (dtype == LA_BF16) return launch_both<__bf16>(b, st);
+    if (dtype == LA_FP16) return launch_both<_Float16>(b, st);
+    return LA_E_UNSUPPORTED;
 }
 
 // Between kCollect and kApply: turns the states the chunks end with (each computed from zero) into the

@@ -83,5 +83,30 @@ def require_gpu(t, what):
         )
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr(device):
+    """hipStream_t of torch's current stream on `device`, as an integer."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)  # no Stream object in between
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def on_device(device):
+    """Context in which `device` is the current HIP device (the library launches on the current one):
+    nothing to do, and nothing done, when it already is."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(device)

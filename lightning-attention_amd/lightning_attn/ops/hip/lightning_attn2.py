@@ -65,7 +65,8 @@ def _fwd(q, k, v, s):
     b, h, n, d = q.shape
     e = v.shape[-1]
     if s is not None:
-        s = s.to(device=q.device, dtype=torch.float32).contiguous()
+        if s.dtype != torch.float32 or s.device != q.device or not s.is_contiguous():
+            s = s.to(device=q.device, dtype=torch.float32).contiguous()
         if s.numel() != h:
             raise ValueError("s must hold one rate per head (%d), got %d" % (h, s.numel()))
     L = _lib.lib()
@@ -75,7 +76,7 @@ def _fwd(q, k, v, s):
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
     sp = s.data_ptr() if s is not None else None
     wp = ws.data_ptr() if ws is not None else None
-    with torch.cuda.device(q.device):
+    with _lib.on_device(q.device):
         if all(t.is_contiguous() for t in (q, k, v, o)):
             rc = L.la_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, o.data_ptr(), b, h, n, d, e, code, wp, ws_bytes,
                           _lib.stream_ptr(q.device))
@@ -99,7 +100,7 @@ def _bwd(q, k, v, s, do):
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
     sp = s.data_ptr() if s is not None else None
     wp = ws.data_ptr() if ws is not None else None
-    with torch.cuda.device(q.device):
+    with _lib.on_device(q.device):
         if all(t.is_contiguous() for t in (q, k, v, do, dq, dk, dv)):
             rc = L.la_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, do.data_ptr(), dq.data_ptr(), dk.data_ptr(),
                           dv.data_ptr(), b, h, n, d, e, code, wp, ws_bytes, _lib.stream_ptr(q.device))

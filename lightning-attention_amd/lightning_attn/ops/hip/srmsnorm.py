@@ -22,7 +22,7 @@ class _SrmsNorm(torch.autograd.Function):
         y = torch.empty_like(x_arg)
         rstd = torch.empty((rows,), dtype=torch.float32, device=x.device)
         L = _lib.lib()
-        with torch.cuda.device(x.device):
+        with _lib.on_device(x.device):
             rc = L.srmsnorm_fwd(x_arg.data_ptr(), y.data_ptr(), rstd.data_ptr(), rows, cols, x_arg.stride(0) if rows else cols,
                                 float(eps), _lib.dtype_code(x.dtype), _lib.stream_ptr(x.device))
         _lib.check(rc, "srmsnorm_fwd")
@@ -44,7 +44,7 @@ class _SrmsNorm(torch.autograd.Function):
         )
         dx = torch.empty_like(dy)
         L = _lib.lib()
-        with torch.cuda.device(x.device):
+        with _lib.on_device(x.device):
             rc = L.srmsnorm_bwd(x_arg.data_ptr(), dy.data_ptr(), rstd.data_ptr(), dx.data_ptr(), rows, cols,
                                 x_arg.stride(0) if rows else cols, _lib.dtype_code(x.dtype), _lib.stream_ptr(x.device))
         _lib.check(rc, "srmsnorm_bwd")

@@ -333,6 +333,39 @@ def test_paired_backward_launch_matches_separate_launches(b, h, n, d, monkeypatc
         check(got["wide"], want, torch.bfloat16, "wide pair d=%d" % d)
 
 
+@pytest.mark.parametrize("b, h, n, d", [(2, 12, 2048, 192), (1, 8, 1024, 128), (2, 3, 777, 64), (1, 2, 300, 256), (1, 5, 913, 72),
+                                        (3, 3, 450, 160), (1, 1, 64, 8), (12, 8, 200, 128)])
+@pytest.mark.parametrize("decay", [True, False])
+def test_backward_in_one_launch(b, h, n, d, decay, monkeypatch):
+    """With d == e and few sequences dQ (walking forward) and dK + dV (walking backward) travel in ONE
+    launch and run side by side; LA_SWEEP_ONCE=0 keeps them apart, =1 joins them whatever the size.
+    Same numbers, bit for bit, for every chunk count, on plain and token-major tensors."""
+    g = torch.Generator().manual_seed(n + d)
+    q, k, v, do = ((torch.randn(b, n, h, d, generator=g) * sc).bfloat16().to(DEV) for sc in (0.7, 0.7, 1.0, 1.0))
+    s = _build_slope_tensor(h) if decay else None
+    monkeypatch.setenv("LA_SWEEP_SCAN", "0")  # (scanned chunk states agree to rounding only)
+    got = {}
+    for token_major in (False, True):
+        tq, tk, tv, tdo = ((t.transpose(1, 2) if token_major else t.transpose(1, 2).contiguous()) for t in (q, k, v, do))
+        for once, chunks in (("0", None), ("1", None), ("1", "1"), ("1", "3"), ("1", "8")):
+            monkeypatch.setenv("LA_SWEEP_ONCE", once)
+            if chunks is None:
+                monkeypatch.delenv("LA_SWEEP_CHUNKS", raising=False)
+            else:
+                monkeypatch.setenv("LA_SWEEP_CHUNKS", chunks)
+            got[token_major, once, chunks] = run_hip(tq.detach(), tk.detach(), tv.detach(), s, tdo)
+    monkeypatch.delenv("LA_SWEEP_ONCE", raising=False)
+    monkeypatch.delenv("LA_SWEEP_CHUNKS", raising=False)
+    got[False, None, None] = run_hip(q.transpose(1, 2).contiguous(), k.transpose(1, 2).contiguous(), v.transpose(1, 2).contiguous(), s,
+                                     do.transpose(1, 2).contiguous())  # the library's own choice
+    monkeypatch.delenv("LA_SWEEP_SCAN", raising=False)
+    for key, val in got.items():
+        for a, c in zip(val, got[False, "0", None]):
+            assert torch.equal(a, c), key
+    want = oracle.linear_attn_fwd_bwd(*(t.transpose(1, 2).cpu() for t in (q, k, v)), s, do.transpose(1, 2).cpu(), torch.float32)
+    check(got[True, "1", "3"], want, torch.bfloat16, "one launch %s" % ((b, h, n, d),))
+
+
 @pytest.mark.parametrize("dtype, decay", [(torch.bfloat16, True), (torch.float16, True), (torch.bfloat16, False)])
 def test_many_sequences_take_the_128_column_workgroups(dtype, decay):
     """b * h >= the number of CUs: the library picks 128-column workgroups for every launch by itself."""

@@ -18,7 +18,7 @@ from oracle import linear_attn_oracle as oracle  # noqa: E402
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
-KNOBS = ("LA_SWEEP_WIDE", "LA_SWEEP_CHUNKS", "LA_SWEEP_UNPAIRED", "LA_SWEEP_SCAN")
+KNOBS = ("LA_SWEEP_WIDE", "LA_SWEEP_CHUNKS", "LA_SWEEP_UNPAIRED", "LA_SWEEP_SCAN", "LA_SWEEP_ONCE")
 
 
 def _rel(a, r):
@@ -45,6 +45,8 @@ def test_random_cases_match_the_oracle(seed, monkeypatch):
             env["LA_SWEEP_SCAN"] = "0"
         if rnd.random() < 0.2:
             env["LA_SWEEP_UNPAIRED"] = "1"
+        if rnd.random() < 0.5:
+            env["LA_SWEEP_ONCE"] = rnd.choice(["0", "1"])
         for name in KNOBS:
             monkeypatch.delenv(name, raising=False)
         for name, value in env.items():
