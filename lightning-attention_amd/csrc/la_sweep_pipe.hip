@@ -707,12 +707,22 @@ __global__ __launch_bounds__(256) void la_state_scan_kernel(float* state, const 
     if (q >= quartets) return;
     const float rate = s ? s[(set / sets_per_unit) % h] : 0.f;
     f32x4* slot = reinterpret_cast<f32x4*>(state) + set * (int64_t)(nchunk - 1) * quartets + q;
+    // every chunk but the last is chunk_len blocks long
+    const float f = s ? expf(-rate * 64.f * (float)chunk_len) : 1.f;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int c = 0; c + 1 < nchunk; ++c) {
-        const int64_t b0 = min((int64_t)c * chunk_len, nblk), b1 = min((int64_t)(c + 1) * chunk_len, nblk);
-        const float f = s ? expf(-rate * 64.f * (float)(b1 - b0)) : 1.f;
-        acc = acc * f + slot[(int64_t)c * quartets];
-        slot[(int64_t)c * quartets] = acc;
+    // the loads of a batch are independent of the running sum: one memory round trip per batch, not per chunk
+    constexpr int BATCH = 16;
+    for (int c0 = 0; c0 + 1 < nchunk; c0 += BATCH) {
+        f32x4 loc[BATCH];
+#pragma unroll
+        for (int i = 0; i < BATCH; ++i)
+            if (c0 + i + 1 < nchunk) loc[i] = slot[(int64_t)(c0 + i) * quartets];
+#pragma unroll
+        for (int i = 0; i < BATCH; ++i)
+            if (c0 + i + 1 < nchunk) {
+                acc = acc * f + loc[i];
+                slot[(int64_t)(c0 + i) * quartets] = acc;
+            }
     }
 }
 
