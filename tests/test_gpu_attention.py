@@ -103,7 +103,8 @@ def test_unit_variance_bf16(b, h, n, d, e, decay):
     check(run_hip(q, k, v, s, do), want, torch.bfloat16, "N(0,1) %s" % ((b, h, n, d, e, decay),))
 
 
-@pytest.mark.parametrize("b, h, n, d, e", [(1, 8, 1024, 64, 64), (2, 3, 333, 128, 128), (1, 4, 130, 16, 40), (1, 2, 64, 8, 8)])
+@pytest.mark.parametrize("b, h, n, d, e", [(1, 8, 1024, 64, 64), (2, 3, 333, 128, 128), (1, 4, 130, 16, 40), (1, 2, 64, 8, 8),
+                                           (1, 2, 200, 96, 128), (1, 3, 257, 128, 72), (2, 2, 100, 32, 64), (1, 1, 70, 72, 104)])
 @pytest.mark.parametrize("decay", [True, False])
 def test_float32(b, h, n, d, e, decay):
     """Config 1's shape (b1 h8 n1024 d=e=64, fp32, slopes(8)) and neighbours: 1e-4 relative."""
