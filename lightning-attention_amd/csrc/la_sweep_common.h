@@ -99,7 +99,7 @@ struct SweepPair {
     SweepArgs a[2];
     int nprod;  // 1 or 2 sweeps; a[1] is unused when 1
     int wide;   // pipelined kernel only: a workgroup covers 128 instead of 64 columns of z / out
-    // Pipelined kernel only.  How a chunk's workgroup gets the state its chunk starts from:
+    // How a chunk's workgroup gets the state its chunk starts from:
     //   kWarmUp   it walks the blocks before its chunk with the state update only (no workspace);
     //   kCollect  first of three launches: every workgroup walks its own chunk, state update only, starting
     //             from zero, and leaves the state it ends with in `state` (the last chunk has nothing to leave);
