@@ -231,6 +231,18 @@ def main():
         q, k, v, do = (torch.randn(b4, h4, n4, d4, device=dev).bfloat16() for _ in range(4))
         q, k, v = q.requires_grad_(), k.requires_grad_(), v.requires_grad_()
         extra["b2_h12_n2048_d192_ms"] = round(event_ms(lambda: (lightning_attn_func(q, k, v, s4).backward(do), _clear(q, k, v)), 30), 4)
+        # the same shape with the C entry points called directly: the two launches of a step without
+        # torch's autograd engine in between (its hand-over to the backward thread bounds the figure above)
+        o4, dq4, dk4, dv4 = (torch.empty_like(q) for _ in range(4))
+
+        def direct4():
+            rc = L.la_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s4.data_ptr(), o4.data_ptr(), b4, h4, n4, d4, d4, 0, None, 0, st)
+            rc = rc or L.la_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s4.data_ptr(), do.data_ptr(), dq4.data_ptr(),
+                                dk4.data_ptr(), dv4.data_ptr(), b4, h4, n4, d4, d4, 0, None, 0, st)
+            assert rc == 0, rc
+
+        extra["b2_h12_n2048_d192_la_fwd_la_bwd_ms"] = round(event_ms(direct4, 30), 4)
+        o4 = dq4 = dk4 = dv4 = None
         extra["b2_h12_n2048_d192_no_decay_ms"] = round(event_ms(lambda: (lightning_attn_func(q, k, v, None).backward(do), _clear(q, k, v)), 30), 4)
         qt, kt, vt = (torch.randn(b4, n4, h4, d4, device=dev).bfloat16().transpose(1, 2).requires_grad_() for _ in range(3))
         dot = torch.randn(b4, n4, h4, d4, device=dev).bfloat16().transpose(1, 2)
