@@ -1,4 +1,6 @@
 // extern "C" entry points of the attention path (see include/lightning_attn_hip.h).
+#include <stdlib.h>
+
 #include <algorithm>
 
 #include "la_sweep_common.h"
@@ -14,6 +16,8 @@ int sweep2(const SweepIO& io0, const SweepIO& io1, const float* s, int64_t bh, i
 size_t sweep_workspace_bytes(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int dtype);
 int sweep_f32(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
               int64_t n, int64_t dk, int64_t dv, bool reverse, hipStream_t st);
+int sweep_f32_bwd_once(const void* q, const void* k, const void* v, const void* dout, void* dq, void* dk, void* dv,
+                       const float* s, int64_t bh, int64_t h, int64_t n, int64_t d, hipStream_t st);
 
 // A tensor argument: device pointer + where its (batch, head, token) rows start.
 struct Tensor {
@@ -100,6 +104,13 @@ static int bwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s
         if ((rc = check_tensor(*ts[i], b, h, n, cols[i], dtype)) != LA_OK) return rc;
     // dQ_i = sum_{j<=i} lam^(i-j) (dO_i . v_j) k_j
     // (the launches follow each other on one stream, so they can all use the same scratch memory)
+    if (d == e && dtype == LA_FP32 && !getenv("LA_SWEEP_UNPAIRED")) {
+        // float32: the three sweeps always share a launch (plain tensors only, as in run())
+        for (int i = 0; i < 7; ++i)
+            if (!is_dense(*ts[i], h, n, d)) return LA_E_UNSUPPORTED;
+        return sweep_f32_bwd_once(q.p, k.p, v.p, dout.p, const_cast<void*>(dq.p), const_cast<void*>(dk.p),
+                                  const_cast<void*>(dv.p), s, b * h, h, n, d, st);
+    }
     if (d == e && dtype != LA_FP32) {
         // few sequences: all three gradients in one launch, side by side (LA_E_UNSUPPORTED: not this time)
         rc = sweep_bwd_once(io(dout, v, k, dq), io(v, dout, q, dk), io(k, q, dout, dv), s, b * h, h, n, d, dtype, ws.p,

@@ -552,11 +552,9 @@ static int64_t warm_up_chunks(int64_t wgs, int64_t nblk) {
     return c > 8 ? 8 : c < 1 ? 1 : c;
 }
 
-static void choose_chunks(SweepArgs& a, int nprod = 1) {
+void plan_warm_up_chunks(int64_t wgs, int64_t nblk, int* nchunk, int* chunk_start /* [9] */) {
     const char* env = getenv("LA_SWEEP_CHUNKS");  // read per call so that tests can vary it
     const int forced = env ? atoi(env) : 0;
-    const int64_t nblk = (a.n + 63) / 64;
-    const int64_t wgs = (int64_t)((a.bh + 7) / 8 * 8) * a.nslice * nprod;
     int64_t c = forced > 0 ? forced : warm_up_chunks(wgs, nblk);
     if (c > 8) c = 8;
     if (c > nblk) c = nblk;
@@ -568,7 +566,7 @@ static void choose_chunks(SweepArgs& a, int nprod = 1) {
     int64_t start = 0;
     wgt = 1.0;
     for (int i = 0; i < c; ++i) {
-        a.chunk_start[i] = (int)start;
+        chunk_start[i] = (int)start;
         int64_t len = (int64_t)((double)nblk * wgt / wsum + 0.5);
         const int64_t left_after = c - 1 - i;
         if (len < 1) len = 1;
@@ -576,9 +574,12 @@ static void choose_chunks(SweepArgs& a, int nprod = 1) {
         start += len;
         wgt *= 1.0 - rho;
     }
-    a.nchunk = (int)c;
-    a.chunk_start[c] = (int)nblk;
-    for (int i = (int)c + 1; i < 9; ++i) a.chunk_start[i] = (int)nblk;
+    *nchunk = (int)c;
+    for (int i = (int)c; i < 9; ++i) chunk_start[i] = (int)nblk;
+}
+
+static void choose_chunks(SweepArgs& a, int nprod = 1) {
+    plan_warm_up_chunks((int64_t)((a.bh + 7) / 8 * 8) * a.nslice * nprod, (a.n + 63) / 64, &a.nchunk, a.chunk_start);
 }
 
 static SweepArgs make_args(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv) {

@@ -29,14 +29,23 @@ struct SweepArgsF32 {
     const float* s;
     int64_t n;
     int dk, dv, h, bh, nslice;
+    // sequence chunks (few sequences): the workgroup of chunk c produces the blocks chunk_start[c] ..
+    // chunk_start[c + 1] - 1 of the walk, after running over the blocks before them with the state
+    // update alone (no workspace, same results bit for bit)
+    int nchunk;
+    int chunk_start[9];
 };
+
+// count and first blocks of the warm-up chunks for `wgs` single-chunk workgroups (la_sweep.hip)
+void plan_warm_up_chunks(int64_t wgs, int64_t nblk, int* nchunk, int* chunk_start);
 
 __device__ __forceinline__ f32x4 mma4(float a, float b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
 }
 
+// `bid`: number of the workgroup within its part of the launch.
 template <int DKP, bool REVERSE, bool DECAY>
-__global__ __launch_bounds__(256, 1) void la_sweep_f32_kernel(SweepArgsF32 a) {
+__device__ __forceinline__ void sweep_f32_body(const SweepArgsF32& a, const unsigned bid) {
     constexpr int XS = DKP + LA_F32_XPAD;  // row stride (floats) of the x / y tiles
     constexpr int ZS = 64 + 4;    // row stride of the z slice and the P tile
     constexpr int KT = DKP / 16;  // 16-row state tiles
@@ -48,9 +57,11 @@ __global__ __launch_bounds__(256, 1) void la_sweep_f32_kernel(SweepArgsF32 a) {
     float* Zs = Ys + 64 * XS;
     float* Ps = Zs + 64 * ZS;
 
-    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-    const int unit = xcd + 8 * (local / a.nslice);
-    const int slice = local % a.nslice;
+    const int xcd = bid & 7, local = bid >> 3;
+    const int per_unit = a.nslice * a.nchunk;
+    const int unit = xcd + 8 * (local / per_unit);
+    const int slice = (local % per_unit) % a.nslice;
+    const int chunk = (local % per_unit) / a.nslice;
     if (unit >= a.bh) return;
 
     const int tid = threadIdx.x;
@@ -90,16 +101,19 @@ __global__ __launch_bounds__(256, 1) void la_sweep_f32_kernel(SweepArgsF32 a) {
     for (int kt = 0; kt < KT; ++kt) st[kt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
     const int64_t nblk = (n + 63) / 64;
+    const int64_t it_first = a.chunk_start[chunk], it_end = a.chunk_start[chunk + 1];
     uint4 xr[XC], yr[XC], zr[4];
 
-    auto load_block = [&](int64_t t) {
-        const int64_t tok0 = t * 64;
+    // block number `it` of the walk; x is not needed for a warm-up block
+    auto load_block = [&](int64_t it) {
+        const int64_t tok0 = (REVERSE ? nblk - 1 - it : it) * 64;
+        const bool need_x = it >= it_first;
 #pragma unroll
         for (int u = 0; u < XC; ++u) {
             const int c = tid + 256 * u;
             const int row = c / (DKP / 4), col = (c % (DKP / 4)) * 4;
             const bool ok = (tok0 + row < n) && (col < dk);
-            xr[u] = ok ? *reinterpret_cast<const uint4*>(xg + (tok0 + row) * dk + col) : make_uint4(0, 0, 0, 0);
+            xr[u] = ok && need_x ? *reinterpret_cast<const uint4*>(xg + (tok0 + row) * dk + col) : make_uint4(0, 0, 0, 0);
             yr[u] = ok ? *reinterpret_cast<const uint4*>(yg + (tok0 + row) * dk + col) : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
@@ -127,19 +141,20 @@ __global__ __launch_bounds__(256, 1) void la_sweep_f32_kernel(SweepArgsF32 a) {
     };
 
     for (int c = tid; c < 64 * ZS / 4; c += 256) reinterpret_cast<uint4*>(Ps)[c] = make_uint4(0, 0, 0, 0);
-    load_block(REVERSE ? nblk - 1 : 0);
+    load_block(0);
     stage_block();
     __syncthreads();
 
     const int jlo = REVERSE ? w : 0, jhi = REVERSE ? 3 : w;
 
-    for (int64_t it = 0; it < nblk; ++it) {
+    for (int64_t it = 0; it < it_end; ++it) {
         const int64_t t = REVERSE ? nblk - 1 - it : it;
-        const bool have_next = it + 1 < nblk;
-        if (have_next) load_block(REVERSE ? t - 1 : t + 1);
+        const bool have_next = it + 1 < it_end;
+        const bool warm = it < it_first;  // warm-up block: state update only
+        if (have_next) load_block(it + 1);
 
         // 1. S^T tiles (rows j, columns i in [16w, 16w+16)) -> masked, decayed P[i][j]
-        {
+        if (!warm) {
             f32x4 sacc[4];
 #pragma unroll
             for (int jt = 0; jt < 4; ++jt) sacc[jt] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -178,6 +193,7 @@ __global__ __launch_bounds__(256, 1) void la_sweep_f32_kernel(SweepArgsF32 a) {
             f32x4 oacc[4];
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
+                if (warm) continue;  // (block-uniform) no output from a warm-up block
                 oacc[i4] = (f32x4){0.f, 0.f, 0.f, 0.f};
                 // 2a. inter-block: st[4K + q][v] holds row 4g + v of its tile, feature 64K + 16v + 4g + q
 #pragma unroll
@@ -208,7 +224,7 @@ __global__ __launch_bounds__(256, 1) void la_sweep_f32_kernel(SweepArgsF32 a) {
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
                 const int64_t tok = t * 64 + 16 * i4 + r;
-                if (tok < n && col < dv) *reinterpret_cast<f32x4*>(og + tok * dv + col) = oacc[i4];
+                if (!warm && tok < n && col < dv) *reinterpret_cast<f32x4*>(og + tok * dv + col) = oacc[i4];
             }
             // 3. state = lam^64 state + y^T (z * Lupd)
             if (have_next) {
@@ -245,6 +261,38 @@ __global__ __launch_bounds__(256, 1) void la_sweep_f32_kernel(SweepArgsF32 a) {
     }
 }
 
+// (70 KB of LDS at DKP = 64: two workgroups fit a CU when the registers do, which the second bound asks for)
+template <int DKP, bool REVERSE, bool DECAY>
+__global__ __launch_bounds__(256, DKP <= 64 ? 2 : 1) void la_sweep_f32_kernel(SweepArgsF32 a) {
+    sweep_f32_body<DKP, REVERSE, DECAY>(a, blockIdx.x);
+}
+
+// The three sweeps of a backward pass with d == e in one launch: part 0 walks forward (dQ), parts 1 and 2
+// backward (dK, dV); the parts have the same number of workgroups (a multiple of 8).
+struct SweepTrioF32 {
+    SweepArgsF32 a[3];
+    unsigned per_part;
+};
+template <int DKP, bool DECAY>
+__global__ __launch_bounds__(256, DKP <= 64 ? 2 : 1) void la_sweep_f32_trio_kernel(SweepTrioF32 t) {
+    const unsigned part = blockIdx.x / t.per_part, bid = blockIdx.x % t.per_part;
+    if (part == 0) sweep_f32_body<DKP, false, DECAY>(t.a[0], bid);
+    else sweep_f32_body<DKP, true, DECAY>(t.a[part == 1 ? 1 : 2], bid);
+}
+
+template <int DKP, bool DECAY>
+static int launch_trio_f32(const SweepTrioF32& t, hipStream_t st) {
+    constexpr size_t lds = (size_t)(2 * 64 * (DKP + LA_F32_XPAD) + 2 * 64 * 68) * sizeof(float);
+    auto kern = la_sweep_f32_trio_kernel<DKP, DECAY>;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+    }
+    hipLaunchKernelGGL(kern, dim3(3 * t.per_part), dim3(256), lds, st, t);
+    return (int)hipGetLastError();
+}
+
 template <int DKP, bool REVERSE, bool DECAY>
 static int launch_one_f32(const SweepArgsF32& a, hipStream_t st) {
     constexpr size_t lds = (size_t)(2 * 64 * (DKP + LA_F32_XPAD) + 2 * 64 * 68) * sizeof(float);
@@ -255,7 +303,7 @@ static int launch_one_f32(const SweepArgsF32& a, hipStream_t st) {
         if (e != hipSuccess) return (int)e;
     }
     const int units8 = (a.bh + 7) / 8 * 8;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(units8 * a.nslice)), dim3(256), lds, st, a);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(units8 * a.nslice * a.nchunk)), dim3(256), lds, st, a);
     return (int)hipGetLastError();
 }
 
@@ -268,15 +316,44 @@ static int launch_dir_f32(const SweepArgsF32& a, hipStream_t st) {
 #undef LA_GO
 }
 
-int sweep_f32(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
-              int64_t n, int64_t dk, int64_t dv, bool reverse, hipStream_t st) {
-    if (dk > 128) return LA_E_UNSUPPORTED;
+static SweepArgsF32 make_args_f32(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
+                                  int64_t n, int64_t dk, int64_t dv) {
     SweepArgsF32 a;
     a.x = static_cast<const float*>(x); a.y = static_cast<const float*>(y); a.z = static_cast<const float*>(z);
     a.out = static_cast<float*>(out); a.s = s;
     a.n = n; a.dk = (int)dk; a.dv = (int)dv; a.h = (int)h; a.bh = (int)bh;
     a.nslice = (int)((dv + 63) / 64);
+    a.nchunk = 1;
+    for (int i = 0; i < 9; ++i) a.chunk_start[i] = i == 0 ? 0 : (int)((n + 63) / 64);
+    return a;
+}
+
+int sweep_f32(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
+              int64_t n, int64_t dk, int64_t dv, bool reverse, hipStream_t st) {
+    if (dk > 128) return LA_E_UNSUPPORTED;
+    SweepArgsF32 a = make_args_f32(x, y, z, out, s, bh, h, n, dk, dv);
+    plan_warm_up_chunks((bh + 7) / 8 * 8 * a.nslice, (n + 63) / 64, &a.nchunk, a.chunk_start);
     return reverse ? launch_dir_f32<true>(a, st) : launch_dir_f32<false>(a, st);
+}
+
+// float32 backward pass with d == e: dQ = fwd(dO, v, k), dK = rev(v, dO, q), dV = rev(k, q, dO) in one
+// launch (the sweeps are independent; with few sequences they run side by side).
+int sweep_f32_bwd_once(const void* q, const void* k, const void* v, const void* dout, void* dq, void* dk, void* dv,
+                       const float* s, int64_t bh, int64_t h, int64_t n, int64_t d, hipStream_t st) {
+    if (d > 128) return LA_E_UNSUPPORTED;
+    SweepTrioF32 t;
+    t.a[0] = make_args_f32(dout, v, k, dq, s, bh, h, n, d, d);
+    t.a[1] = make_args_f32(v, dout, q, dk, s, bh, h, n, d, d);
+    t.a[2] = make_args_f32(k, q, dout, dv, s, bh, h, n, d, d);
+    plan_warm_up_chunks((bh + 7) / 8 * 8 * t.a[0].nslice * 3, (n + 63) / 64, &t.a[0].nchunk, t.a[0].chunk_start);
+    for (int i = 1; i < 3; ++i) {
+        t.a[i].nchunk = t.a[0].nchunk;
+        for (int j = 0; j < 9; ++j) t.a[i].chunk_start[j] = t.a[0].chunk_start[j];
+    }
+    t.per_part = (unsigned)((bh + 7) / 8 * 8 * t.a[0].nslice * t.a[0].nchunk);
+    const bool decay = s != nullptr;
+    if (d <= 64) return decay ? launch_trio_f32<64, true>(t, st) : launch_trio_f32<64, false>(t, st);
+    return decay ? launch_trio_f32<128, true>(t, st) : launch_trio_f32<128, false>(t, st);
 }
 
 }  // namespace la

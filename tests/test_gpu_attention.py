@@ -116,6 +116,28 @@ def test_float32(b, h, n, d, e, decay):
     check(run_hip(q, k, v, s, do), want, torch.float32, "fp32 %s" % ((b, h, n, d, e, decay),))
 
 
+@pytest.mark.parametrize("b, h, n, d", [(1, 8, 1024, 64), (2, 3, 333, 128), (3, 5, 70, 24), (1, 1, 200, 96)])
+@pytest.mark.parametrize("decay", [True, False])
+def test_float32_backward_in_one_launch(b, h, n, d, decay, monkeypatch):
+    """float32 with d == e: dQ, dK and dV share a launch; LA_SWEEP_UNPAIRED=1 launches them one after
+    the other.  Same numbers, bit for bit."""
+    q, k, v, do = make_inputs(b, h, n, d, d, torch.float32, 1.0, seed=n)
+    s = _build_slope_tensor(h) if decay else None
+    together = run_hip(q, k, v, s, do)
+    monkeypatch.setenv("LA_SWEEP_UNPAIRED", "1")
+    apart = run_hip(q, k, v, s, do)
+    monkeypatch.delenv("LA_SWEEP_UNPAIRED", raising=False)
+    for a, c in zip(together, apart):
+        assert torch.equal(a, c)
+    # few sequences: the walk is cut into chunks with warm-up blocks, here as well bit-identical for every count
+    for chunks in ("1", "2", "5", "8"):
+        monkeypatch.setenv("LA_SWEEP_CHUNKS", chunks)
+        for a, c in zip(run_hip(q, k, v, s, do), together):
+            assert torch.equal(a, c), chunks
+    monkeypatch.delenv("LA_SWEEP_CHUNKS", raising=False)
+    check(together, oracle.linear_attn_fwd_bwd(q, k, v, s, do, torch.float64), torch.float32, "fp32 one launch")
+
+
 def test_config4_d192_decay_and_zero_rates():
     """b2 h12 n2048 d=e=192: slopes(12) (non power of two head count), s=None and s=0 agree."""
     b, h, n, d, e = 2, 12, 2048, 192, 192
