@@ -122,6 +122,10 @@ struct SweepBoth {
 };
 int sweep_pipe_both(const SweepBoth& b, int dtype, hipStream_t st);  // feature dim up to 128, la_sweep_pipe.hip
 
+// Count (up to 8) and first blocks, chunk_start[0 .. 8], of the warm-up chunks for a launch that would have
+// `wgs` workgroups with one chunk each, on a walk of nblk blocks; defined in la_sweep.hip.
+void plan_warm_up_chunks(int64_t wgs, int64_t nblk, int* nchunk, int* chunk_start);
+
 // Launches the single-barrier pipelined kernel (feature dim up to 128); defined in la_sweep_pipe.hip.
 // n, dk, dv, h, bh, nslice and the chunking must agree between the two sweeps of a pair.
 enum { kWarmUp = 0, kCollect = 1, kApply = 2 };

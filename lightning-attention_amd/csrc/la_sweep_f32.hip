@@ -12,7 +12,7 @@
 //   state tiles   come in groups of four (kt = 4K + q); row rho of tile kt is feature
 //                 64K + 4 pi(rho) + q with pi(rho) = 4 (rho % 4) + rho / 4, so that one 16-byte read of a
 //                 y row (state update) or an x row (inter-block term) feeds the four tiles of a group.
-#include "la_common.h"
+#include "la_sweep_common.h"
 #include "lightning_attn_hip.h"
 
 namespace la {
@@ -36,8 +36,6 @@ struct SweepArgsF32 {
     int chunk_start[9];
 };
 
-// count and first blocks of the warm-up chunks for `wgs` single-chunk workgroups (la_sweep.hip)
-void plan_warm_up_chunks(int64_t wgs, int64_t nblk, int* nchunk, int* chunk_start);
 
 __device__ __forceinline__ f32x4 mma4(float a, float b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
