@@ -11,6 +11,8 @@ int sweep(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, i
           bool reverse, void* ws, size_t ws_bytes, hipStream_t st);
 int sweep_bwd_once(const SweepIO& dq, const SweepIO& dk, const SweepIO& dv, const float* s, int64_t bh, int64_t h, int64_t n,
                    int64_t d, int dtype, void* ws, size_t ws_bytes, hipStream_t st);
+int sweep_fwd_rev_once(const SweepIO& fwd, const SweepIO& rev, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk,
+                       int64_t dv, int dtype, void* ws, size_t ws_bytes, hipStream_t st);
 int sweep2(const SweepIO& io0, const SweepIO& io1, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv,
            int dtype, bool reverse, void* ws, size_t ws_bytes, hipStream_t st);
 size_t sweep_workspace_bytes(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int dtype);
@@ -115,6 +117,12 @@ static int bwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s
         // few sequences: all three gradients in one launch, side by side (LA_E_UNSUPPORTED: not this time)
         rc = sweep_bwd_once(io(dout, v, k, dq), io(v, dout, q, dk), io(k, q, dout, dv), s, b * h, h, n, d, dtype, ws.p,
                             ws.bytes, st);
+        if (rc != LA_E_UNSUPPORTED) return rc;
+    }
+    if (d != e && dtype != LA_FP32) {
+        // dQ and dK have one shape and opposite directions: with few sequences, one launch for the two
+        rc = sweep_fwd_rev_once(io(dout, v, k, dq), io(v, dout, q, dk), s, b * h, h, n, e, d, dtype, ws.p, ws.bytes, st);
+        if (rc == LA_OK) return run(k, q, dout, dv, s, b * h, h, n, d, e, dtype, true, ws, st);
         if (rc != LA_E_UNSUPPORTED) return rc;
     }
     rc = run(dout, v, k, dq, s, b * h, h, n, e, d, dtype, false, ws, st);

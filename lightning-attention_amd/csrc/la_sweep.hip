@@ -803,4 +803,45 @@ int sweep_bwd_once(const SweepIO& dq, const SweepIO& dk, const SweepIO& dv, cons
     return launch_both<_Float16>(b, st);
 }
 
+// The same for two sweeps of one shape and opposite directions (dQ and dK of a backward pass with
+// d != e: both contract over e and produce d columns): one launch where they fit on the chip together
+// and separate launches are not estimated faster; LA_E_UNSUPPORTED otherwise.
+int sweep_fwd_rev_once(const SweepIO& fwd, const SweepIO& rev, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk,
+                       int64_t dv, int dtype, void* ws, size_t ws_bytes, hipStream_t st) {
+    if (dtype != LA_BF16 && dtype != LA_FP16) return LA_E_UNSUPPORTED;
+    const char* env = getenv("LA_SWEEP_ONCE");
+    const int forced = env ? (atoi(env) != 0 ? 1 : -1) : 0;
+    if (forced < 0 || getenv("LA_SWEEP_UNPAIRED")) return LA_E_UNSUPPORTED;
+    const char* wide_env = getenv("LA_SWEEP_WIDE");
+    if (forced == 0 && wide_env && atoi(wide_env) != 0) return LA_E_UNSUPPORTED;
+    const int64_t cus = num_cus(), nblk = (n + 63) / 64, nslice = (dv + 63) / 64;
+    const int64_t wgs = (bh + 7) / 8 * 8 * nslice * 2;
+    if (forced == 0) {
+        if (wgs > cus) return LA_E_UNSUPPORTED;
+        const bool ws_ok = ws && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0;
+        const bool wide = wide_columns(bh, n, dk, dv, 1, ws_ok ? ws_bytes : 0);
+        const ScanPlan pl = plan_scan(bh, n, dk, dv, 1, wide);
+        const double separate = 2.0 * (pl.nchunk > 1 && ws_ok && ws_bytes >= pl.bytes ? pl.us : warm_up_us(bh, n, dk, dv, 1, wide));
+        if (warm_up_frac(wgs, nblk) * (double)nblk * block_us(dk, false) >= separate) return LA_E_UNSUPPORTED;
+    }
+    SweepBoth b;
+    b.fwd.nprod = b.rev.nprod = 1;
+    b.fwd.a[0] = make_args(fwd, s, bh, h, n, dk, dv);
+    b.rev.a[0] = make_args(rev, s, bh, h, n, dk, dv);
+    choose_chunks(b.fwd.a[0], 2);
+    b.rev.a[0].nchunk = b.fwd.a[0].nchunk;
+    for (int j = 0; j < 9; ++j) b.rev.a[0].chunk_start[j] = b.fwd.a[0].chunk_start[j];
+    for (SweepPair* p : {&b.fwd, &b.rev}) {
+        p->a[1] = p->a[0];
+        p->wide = 0;
+        p->mode = kWarmUp;
+        p->chunk_len = 0;
+        p->state = nullptr;
+    }
+    b.nfwd = part_grid(b.fwd);
+    if (dk <= 128) return sweep_pipe_both(b, dtype, st);
+    if (dtype == LA_BF16) return launch_both<__bf16>(b, st);
+    return launch_both<_Float16>(b, st);
+}
+
 }  // namespace la

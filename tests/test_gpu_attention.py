@@ -389,6 +389,39 @@ def test_backward_in_one_launch(b, h, n, d, decay, monkeypatch):
     check(got[True, "1", "3"], want, torch.bfloat16, "one launch %s" % ((b, h, n, d),))
 
 
+@pytest.mark.parametrize("b, h, n, d, e", [(2, 8, 1024, 128, 64), (1, 3, 777, 64, 128), (1, 2, 300, 192, 256), (1, 2, 513, 72, 40),
+                                           (2, 2, 1100, 256, 128), (12, 8, 200, 128, 64)])
+@pytest.mark.parametrize("decay", [True, False])
+def test_dq_and_dk_in_one_launch(b, h, n, d, e, decay, monkeypatch):
+    """With d != e the dQ sweep (walking forward) and the dK sweep (walking backward) have one shape
+    and, with few sequences, share a launch; dV follows.  LA_SWEEP_ONCE=0 / 1 as above; same numbers,
+    bit for bit, on plain and token-major tensors."""
+    g = torch.Generator().manual_seed(n + d + e)
+    q, k = ((torch.randn(b, n, h, d, generator=g) * 0.7).bfloat16().to(DEV) for _ in range(2))
+    v, do = (torch.randn(b, n, h, e, generator=g).bfloat16().to(DEV) for _ in range(2))
+    s = _build_slope_tensor(h) if decay else None
+    monkeypatch.setenv("LA_SWEEP_SCAN", "0")
+    got = {}
+    for token_major in (False, True):
+        tq, tk, tv, tdo = ((t.transpose(1, 2) if token_major else t.transpose(1, 2).contiguous()) for t in (q, k, v, do))
+        for once, chunks in (("0", None), ("1", None), ("1", "1"), ("1", "4")):
+            monkeypatch.setenv("LA_SWEEP_ONCE", once)
+            if chunks is None:
+                monkeypatch.delenv("LA_SWEEP_CHUNKS", raising=False)
+            else:
+                monkeypatch.setenv("LA_SWEEP_CHUNKS", chunks)
+            got[token_major, once, chunks] = run_hip(tq.detach(), tk.detach(), tv.detach(), s, tdo)
+    monkeypatch.delenv("LA_SWEEP_ONCE", raising=False)
+    monkeypatch.delenv("LA_SWEEP_CHUNKS", raising=False)
+    got["auto"] = run_hip(*(t.transpose(1, 2).contiguous() for t in (q, k, v)), s, do.transpose(1, 2).contiguous())
+    monkeypatch.delenv("LA_SWEEP_SCAN", raising=False)
+    for key, val in got.items():
+        for a, c in zip(val, got[False, "0", None]):
+            assert torch.equal(a, c), key
+    want = oracle.linear_attn_fwd_bwd(*(t.transpose(1, 2).cpu() for t in (q, k, v)), s, do.transpose(1, 2).cpu(), torch.float32)
+    check(got[True, "1", "4"], want, torch.bfloat16, "dq + dk in one launch %s" % ((b, h, n, d, e),))
+
+
 @pytest.mark.parametrize("dtype, decay", [(torch.bfloat16, True), (torch.float16, True), (torch.bfloat16, False)])
 def test_many_sequences_take_the_128_column_workgroups(dtype, decay):
     """b * h >= the number of CUs: the library picks 128-column workgroups for every launch by itself."""
