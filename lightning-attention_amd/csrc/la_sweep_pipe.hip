@@ -378,7 +378,6 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
     // One iteration.  `xr, yr, zr` hold block it+2 on entry and block it+4 on exit.
     auto iteration = [&](auto role, const int64_t it, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4 (&zr)[ZC]) __attribute__((always_inline)) {
         constexpr bool STATE = decltype(role)::value;
-        const int64_t t = REVERSE ? nblk - 1 - it : it;
         const bool have_next = it + 1 < it_end;
         const bool warm = it < it_first;  // warm-up block: state update only
         const int bcur = (int)((unsigned)it % 3u);
@@ -701,7 +700,7 @@ int sweep_pipe_both(const SweepBoth& b, int dtype, hipStream_t st) {
 // on exit (S_in[0] = 0).  One thread per accumulator quartet, chunks in order; the layout inside a slot
 // does not matter.
 __global__ __launch_bounds__(256) void la_state_scan_kernel(float* state, const float* s, int h, int sets_per_unit,
-                                                           int nchunk, int chunk_len, int64_t nblk, int quartets) {
+                                                           int nchunk, int chunk_len, int quartets) {
     const int q = blockIdx.x * 256 + threadIdx.x;  // quartet within the slot
     const int64_t set = blockIdx.y;                // (unit, sweep, slice)
     if (q >= quartets) return;
@@ -730,9 +729,8 @@ int launch_state_scan(const SweepPair& p, hipStream_t st) {
     const SweepArgs& a = p.a[0];
     const int quartets = (int)(pipe_state_floats(a.dk, p.wide != 0) / 4);
     const int sets_per_unit = p.nprod * a.nslice;
-    const int64_t nblk = (a.n + 63) / 64;
     hipLaunchKernelGGL(la_state_scan_kernel, dim3((unsigned)((quartets + 255) / 256), (unsigned)(a.bh * sets_per_unit)),
-                       dim3(256), 0, st, p.state, a.s, a.h, sets_per_unit, a.nchunk, p.chunk_len, nblk, quartets);
+                       dim3(256), 0, st, p.state, a.s, a.h, sets_per_unit, a.nchunk, p.chunk_len, quartets);
     return (int)hipGetLastError();
 }
 
