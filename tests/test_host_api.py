@@ -83,6 +83,36 @@ def test_host_only_entry_points():
     assert L.srmsnorm_bwd(p16, p16, p16, p16, 0, 64, 64, 0, None) == 0
 
 
+def test_workspace_query_is_consistent(monkeypatch):
+    """Properties of the scratch size over a grid of shapes (host logic only; without a device the library
+    plans for 256 CUs): a whole number of state slots, never more than 63 of them per sequence, sweep and
+    column slice, nothing for float32 or when the sequences fill the chip by themselves, nothing when
+    scanned chunk states are switched off, and the backward pass never asks for less than the forward."""
+    L = _lib.lib()
+    for name in ("LA_SWEEP_WIDE", "LA_SWEEP_CHUNKS", "LA_SWEEP_SCAN", "LA_SWEEP_UNPAIRED", "LA_SWEEP_ONCE"):
+        monkeypatch.delenv(name, raising=False)
+    seen_some = False
+    for b, h in ((1, 1), (1, 8), (2, 12), (1, 32), (4, 32), (8, 64)):
+        for n in (64, 1000, 4096, 65536):
+            for d in (8, 64, 128, 192, 256):
+                for e in (d, 64):
+                    fwd = L.la_workspace_bytes(0, b, h, n, d, e, 0)
+                    bwd = L.la_workspace_bytes(1, b, h, n, d, e, 0)
+                    assert L.la_workspace_bytes(0, b, h, n, min(d, 128), min(e, 128), 2) == 0  # float32
+                    assert fwd % 16 == 0 and bwd % 16 == 0 and bwd >= fwd
+                    # one slot: (feature dim padded to 64 / 128 / 192 / 256) x (64 or 128 columns) floats
+                    cap = lambda dk, dv: b * h * 2 * ((dv + 63) // 64) * 63 * max(128, -(-dk // 64) * 64) * 128 * 4
+                    assert fwd <= cap(d, e) and bwd <= max(cap(e, d), cap(d, e))
+                    if b * h >= 256 or n <= 64:
+                        assert fwd == 0 and bwd == 0
+                    seen_some = seen_some or fwd > 0
+    assert seen_some
+    assert L.la_workspace_bytes(0, 1, 8, 65536, 128, 128, 0) > 0
+    monkeypatch.setenv("LA_SWEEP_SCAN", "0")
+    assert L.la_workspace_bytes(0, 1, 8, 65536, 128, 128, 0) == 0
+    assert L.la_workspace_bytes(1, 1, 8, 65536, 192, 192, 0) == 0
+
+
 def test_no_cpu_fallback():
     q = torch.randn(1, 2, 16, 16)
     with pytest.raises(RuntimeError, match="HIP device"):
