@@ -18,7 +18,9 @@
  *   - dtype: LA_BF16 = 0, LA_FP16 = 1, LA_FP32 = 2 (element type of q,k,v,o and
  *     of the gradients; x,y,dy,dx for the norm).  Slopes, rstd and every
  *     accumulator are float32;
- *   - calls are re-entrant and thread-safe: the library keeps no mutable state.
+ *   - calls are re-entrant and thread-safe: the library keeps no mutable state and reads
+ *     nothing from the process environment; how a call is mapped onto launches depends on
+ *     its arguments alone (la_launch_opts below, where a caller wants to override that).
  */
 #ifndef LIGHTNING_ATTN_HIP_H
 #define LIGHTNING_ATTN_HIP_H
@@ -37,7 +39,7 @@ enum {
     LA_E_NULLPTR = -1,     /* a required pointer is NULL                      */
     LA_E_SHAPE = -2,       /* a dimension is <= 0 or exceeds the index range  */
     LA_E_UNSUPPORTED = -3, /* head dims / dtype outside la_supported()        */
-    LA_E_WORKSPACE = -4,   /* internal: scratch expected but absent            */
+    LA_E_WORKSPACE = -4,   /* workspace too small for the requested plan       */
     LA_E_ALIGN = -5        /* a pointer or stride is not 16-byte aligned      */
 };
 
@@ -55,8 +57,26 @@ int la_supported(int64_t d, int64_t e, int dtype);
  * or fewer bytes than this, the chunks rebuild their incoming state by walking the blocks before
  * them instead, which gives bit-identical results to the single walk and is several times slower
  * for long sequences.  16-byte aligned; contents need not survive the call, and calls that follow
- * each other on one stream may share it. */
+ * each other on one stream may share it.  0 for shapes la_fwd / la_bwd reject. */
 size_t la_workspace_bytes(int which, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype);
+
+/*
+ * How a call is mapped onto kernel launches.  A zero-filled struct (or a NULL pointer where one is
+ * taken) leaves every choice to the library, which is what production callers want; the fields
+ * exist for measurements and for tests that compare the launch forms with each other.  Results
+ * are bit-identical across all settings except `scan` / `chunks` with a workspace (chunk states
+ * summed in another order: equal to rounding).
+ */
+enum { LA_OPT_AUTO = 0, LA_OPT_OFF = 1, LA_OPT_ON = 2 };
+typedef struct la_launch_opts {
+    int32_t chunks; /* sequence chunks per (batch, head, column slice): 0 = library's choice, > 0 forced
+                       (at most 64 from scanned states, 8 with warm-up blocks, never more than blocks) */
+    int32_t scan;   /* start chunks from scanned states in the workspace: LA_OPT_AUTO (where estimated
+                       faster and the workspace suffices) / LA_OPT_OFF (warm-up blocks only)            */
+    int32_t wide;   /* 128 instead of 64 output columns per workgroup (d,e <= 128): AUTO / OFF / ON     */
+    int32_t paired; /* backward, d == e: dK and dV in one launch: AUTO (yes) / OFF (one after the other) */
+    int32_t once;   /* backward, few sequences: every sweep in one launch: AUTO / OFF / ON               */
+} la_launch_opts;
 
 /*
  * Forward of decayed causal linear attention, O = (Q K^T * M_h) V with
@@ -105,6 +125,25 @@ int la_bwd_strided(const void *q, const void *k, const void *v, const float *s, 
                    void *workspace, size_t ws_bytes, void *stream);
 
 /*
+ * The same entry points with explicit launch options: `strides` as in la_fwd_strided /
+ * la_bwd_strided or NULL for plain (b,h,n,d) tensors; `opts` NULL for the library's own choices
+ * (then they are exactly la_fwd / la_bwd / la_fwd_strided / la_bwd_strided / la_workspace_bytes).
+ * A workspace sized by la_workspace_bytes_opts with the same opts is always large enough.
+ * No counterpart in the reference, whose launch shapes are constants
+ * (lightning_attn/ops/triton/lightning_attn2.py:410-414, 454-458).
+ */
+size_t la_workspace_bytes_opts(int which, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
+                               const la_launch_opts *opts);
+int la_fwd_opts(const void *q, const void *k, const void *v, const float *s, void *o,
+                const int64_t *strides,
+                int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
+                void *workspace, size_t ws_bytes, const la_launch_opts *opts, void *stream);
+int la_bwd_opts(const void *q, const void *k, const void *v, const float *s, const void *dout,
+                void *dq, void *dk, void *dv, const int64_t *strides,
+                int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
+                void *workspace, size_t ws_bytes, const la_launch_opts *opts, void *stream);
+
+/*
  * SimpleRMSNorm forward: rstd[r] = 1/sqrt(mean(x[r,:]^2) + eps), y = x * rstd.
  * x,y: rows x cols with `row_stride` elements between rows; rstd: rows floats.
  * Replaces _SrmsNorm.forward + srms_norm_fw
@@ -115,6 +154,8 @@ int srmsnorm_fwd(const void *x, void *y, float *rstd, int64_t rows, int64_t cols
 
 /*
  * SimpleRMSNorm backward: xhat = x*rstd; dx = (dy - xhat*mean(xhat*dy)) * rstd.
+ * Only x has `row_stride`; dy and dx are dense rows x cols arrays (the reference makes dy
+ * contiguous and allocates dx like it, srmsnorm.py:149-151).
  * Replaces _SrmsNorm.backward + srms_norm_bwd_dx_fused
  * (lightning_attn/ops/triton/srmsnorm.py:38-74, 125-175).
  */

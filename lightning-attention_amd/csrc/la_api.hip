@@ -1,6 +1,4 @@
 // extern "C" entry points of the attention path (see include/lightning_attn_hip.h).
-#include <stdlib.h>
-
 #include <algorithm>
 
 #include "la_sweep_common.h"
@@ -8,18 +6,18 @@
 
 namespace la {
 int sweep(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
-          bool reverse, void* ws, size_t ws_bytes, hipStream_t st);
+          bool reverse, void* ws, size_t ws_bytes, const Opts& opts, hipStream_t st);
 int sweep_bwd_once(const SweepIO& dq, const SweepIO& dk, const SweepIO& dv, const float* s, int64_t bh, int64_t h, int64_t n,
-                   int64_t d, int dtype, void* ws, size_t ws_bytes, hipStream_t st);
+                   int64_t d, int dtype, void* ws, size_t ws_bytes, const Opts& opts, hipStream_t st);
 int sweep_fwd_rev_once(const SweepIO& fwd, const SweepIO& rev, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk,
-                       int64_t dv, int dtype, void* ws, size_t ws_bytes, hipStream_t st);
+                       int64_t dv, int dtype, void* ws, size_t ws_bytes, const Opts& opts, hipStream_t st);
 int sweep2(const SweepIO& io0, const SweepIO& io1, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv,
-           int dtype, bool reverse, void* ws, size_t ws_bytes, hipStream_t st);
-size_t sweep_workspace_bytes(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int dtype);
+           int dtype, bool reverse, void* ws, size_t ws_bytes, const Opts& opts, hipStream_t st);
+size_t sweep_workspace_bytes(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int dtype, const Opts& opts);
 int sweep_f32(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
-              int64_t n, int64_t dk, int64_t dv, bool reverse, hipStream_t st);
+              int64_t n, int64_t dk, int64_t dv, bool reverse, int chunks, hipStream_t st);
 int sweep_f32_bwd_once(const void* q, const void* k, const void* v, const void* dout, void* dq, void* dk, void* dv,
-                       const float* s, int64_t bh, int64_t h, int64_t n, int64_t d, hipStream_t st);
+                       const float* s, int64_t bh, int64_t h, int64_t n, int64_t d, int chunks, hipStream_t st);
 
 // A tensor argument: device pointer + where its (batch, head, token) rows start.
 struct Tensor {
@@ -44,14 +42,14 @@ struct Scratch {
 
 // one directional sweep at the element type named by dtype
 static int run(const Tensor& x, const Tensor& y, const Tensor& z, const Tensor& out, const float* s, int64_t bh, int64_t h,
-               int64_t n, int64_t dk, int64_t dv, int dtype, bool reverse, const Scratch& ws, hipStream_t st) {
+               int64_t n, int64_t dk, int64_t dv, int dtype, bool reverse, const Scratch& ws, const Opts& opts, hipStream_t st) {
     if (dtype == LA_FP32) {
         // the float32 accuracy kernel takes plain (b, h, n, d) tensors only
         if (!is_dense(x, h, n, dk) || !is_dense(y, h, n, dk) || !is_dense(z, h, n, dv) || !is_dense(out, h, n, dv))
             return LA_E_UNSUPPORTED;
-        return sweep_f32(x.p, y.p, z.p, const_cast<void*>(out.p), s, bh, h, n, dk, dv, reverse, st);
+        return sweep_f32(x.p, y.p, z.p, const_cast<void*>(out.p), s, bh, h, n, dk, dv, reverse, opts.chunks, st);
     }
-    return sweep(io(x, y, z, out), s, bh, h, n, dk, dv, dtype, reverse, ws.p, ws.bytes, st);
+    return sweep(io(x, y, z, out), s, bh, h, n, dk, dv, dtype, reverse, ws.p, ws.bytes, opts, st);
 }
 
 static inline bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -64,6 +62,14 @@ static int check_dims(int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int
     if (!la_supported(d, e, dtype)) return LA_E_UNSUPPORTED;
     return LA_OK;
 }
+
+static int check_opts(const Opts& o) {
+    if (o.chunks < 0) return LA_E_SHAPE;
+    for (int v : {o.scan, o.wide, o.paired, o.once})
+        if (v != LA_OPT_AUTO && v != LA_OPT_OFF && v != LA_OPT_ON) return LA_E_SHAPE;
+    return LA_OK;
+}
+static const Opts kAuto = {0, LA_OPT_AUTO, LA_OPT_AUTO, LA_OPT_AUTO, LA_OPT_AUTO};
 
 // pointer and strides of one tensor with `cols` features per row
 static int check_tensor(const Tensor& t, int64_t b, int64_t h, int64_t n, int64_t cols, int dtype) {
@@ -79,9 +85,10 @@ static int check_tensor(const Tensor& t, int64_t b, int64_t h, int64_t n, int64_
 }
 
 static int fwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s, const Tensor& o, int64_t b, int64_t h,
-               int64_t n, int64_t d, int64_t e, int dtype, const Scratch& ws, hipStream_t st) {
+               int64_t n, int64_t d, int64_t e, int dtype, const Scratch& ws, const Opts& opts, hipStream_t st) {
     int rc = check_dims(b, h, n, d, e, dtype);
     if (rc != LA_OK) return rc;
+    if ((rc = check_opts(opts)) != LA_OK) return rc;
     if (b == 0 || n == 0) return LA_OK;  // nothing to do; empty tensors may carry null pointers
     const Tensor* ts[4] = {&q, &k, &v, &o};
     const int64_t cols[4] = {d, d, e, e};
@@ -89,14 +96,15 @@ static int fwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s
         if (!ts[i]->p) return LA_E_NULLPTR;
     for (int i = 0; i < 4; ++i)
         if ((rc = check_tensor(*ts[i], b, h, n, cols[i], dtype)) != LA_OK) return rc;
-    return run(q, k, v, o, s, b * h, h, n, d, e, dtype, false, ws, st);
+    return run(q, k, v, o, s, b * h, h, n, d, e, dtype, false, ws, opts, st);
 }
 
 static int bwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s, const Tensor& dout, const Tensor& dq,
                const Tensor& dk, const Tensor& dv, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
-               const Scratch& ws, hipStream_t st) {
+               const Scratch& ws, const Opts& opts, hipStream_t st) {
     int rc = check_dims(b, h, n, d, e, dtype);
     if (rc != LA_OK) return rc;
+    if ((rc = check_opts(opts)) != LA_OK) return rc;
     if (b == 0 || n == 0) return LA_OK;
     const Tensor* ts[7] = {&q, &k, &v, &dout, &dq, &dk, &dv};
     const int64_t cols[7] = {d, d, e, e, d, d, e};
@@ -106,34 +114,34 @@ static int bwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s
         if ((rc = check_tensor(*ts[i], b, h, n, cols[i], dtype)) != LA_OK) return rc;
     // dQ_i = sum_{j<=i} lam^(i-j) (dO_i . v_j) k_j
     // (the launches follow each other on one stream, so they can all use the same scratch memory)
-    if (d == e && dtype == LA_FP32 && !getenv("LA_SWEEP_UNPAIRED")) {
+    if (d == e && dtype == LA_FP32 && opts.paired != LA_OPT_OFF) {
         // float32: the three sweeps always share a launch (plain tensors only, as in run())
         for (int i = 0; i < 7; ++i)
             if (!is_dense(*ts[i], h, n, d)) return LA_E_UNSUPPORTED;
         return sweep_f32_bwd_once(q.p, k.p, v.p, dout.p, const_cast<void*>(dq.p), const_cast<void*>(dk.p),
-                                  const_cast<void*>(dv.p), s, b * h, h, n, d, st);
+                                  const_cast<void*>(dv.p), s, b * h, h, n, d, opts.chunks, st);
     }
     if (d == e && dtype != LA_FP32) {
         // few sequences: all three gradients in one launch, side by side (LA_E_UNSUPPORTED: not this time)
         rc = sweep_bwd_once(io(dout, v, k, dq), io(v, dout, q, dk), io(k, q, dout, dv), s, b * h, h, n, d, dtype, ws.p,
-                            ws.bytes, st);
+                            ws.bytes, opts, st);
         if (rc != LA_E_UNSUPPORTED) return rc;
     }
     if (d != e && dtype != LA_FP32) {
         // dQ and dK have one shape and opposite directions: with few sequences, one launch for the two
-        rc = sweep_fwd_rev_once(io(dout, v, k, dq), io(v, dout, q, dk), s, b * h, h, n, e, d, dtype, ws.p, ws.bytes, st);
-        if (rc == LA_OK) return run(k, q, dout, dv, s, b * h, h, n, d, e, dtype, true, ws, st);
+        rc = sweep_fwd_rev_once(io(dout, v, k, dq), io(v, dout, q, dk), s, b * h, h, n, e, d, dtype, ws.p, ws.bytes, opts, st);
+        if (rc == LA_OK) return run(k, q, dout, dv, s, b * h, h, n, d, e, dtype, true, ws, opts, st);
         if (rc != LA_E_UNSUPPORTED) return rc;
     }
-    rc = run(dout, v, k, dq, s, b * h, h, n, e, d, dtype, false, ws, st);
+    rc = run(dout, v, k, dq, s, b * h, h, n, e, d, dtype, false, ws, opts, st);
     if (rc != LA_OK) return rc;
     // dK_j = sum_{i>=j} lam^(i-j) (v_j . dO_i) q_i   and   dV_j = sum_{i>=j} lam^(i-j) (k_j . q_i) dO_i
     // have the same shape when d == e: one launch, in which they share the reads of dO and q
     if (d == e && dtype != LA_FP32)
-        return sweep2(io(v, dout, q, dk), io(k, q, dout, dv), s, b * h, h, n, d, e, dtype, true, ws.p, ws.bytes, st);
-    rc = run(v, dout, q, dk, s, b * h, h, n, e, d, dtype, true, ws, st);
+        return sweep2(io(v, dout, q, dk), io(k, q, dout, dv), s, b * h, h, n, d, e, dtype, true, ws.p, ws.bytes, opts, st);
+    rc = run(v, dout, q, dk, s, b * h, h, n, e, d, dtype, true, ws, opts, st);
     if (rc != LA_OK) return rc;
-    return run(k, q, dout, dv, s, b * h, h, n, d, e, dtype, true, ws, st);
+    return run(k, q, dout, dv, s, b * h, h, n, d, e, dtype, true, ws, opts, st);
 }
 }  // namespace la
 
@@ -145,7 +153,7 @@ extern "C" const char* la_error_string(int code) {
         case LA_E_NULLPTR: return "a required pointer is NULL";
         case LA_E_SHAPE: return "a dimension is out of range";
         case LA_E_UNSUPPORTED: return "head dims / dtype not supported (need d,e multiples of 8 in [8,256]; [8,128] for float32)";
-        case LA_E_WORKSPACE: return "workspace too small";
+        case LA_E_WORKSPACE: return "workspace too small for the requested plan";
         case LA_E_ALIGN: return "pointer not 16-byte aligned";
         default: break;
     }
@@ -161,52 +169,77 @@ extern "C" int la_supported(int64_t d, int64_t e, int dtype) {
     return 1;
 }
 
-extern "C" size_t la_workspace_bytes(int which, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype) {
-    if (b <= 0 || h <= 0 || n <= 0 || !la_supported(d, e, dtype)) return 0;
+extern "C" size_t la_workspace_bytes_opts(int which, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
+                                          const la_launch_opts* opts) {
+    const la::Opts& o = opts ? *opts : la::kAuto;
+    // nothing for empty tensors and for shapes the entry points reject
+    if (b <= 0 || n <= 0 || la::check_dims(b, h, n, d, e, dtype) != LA_OK || la::check_opts(o) != LA_OK) return 0;
     using la::sweep_workspace_bytes;
     const int64_t bh = b * h;
-    if (which == 0) return sweep_workspace_bytes(bh, n, d, e, 1, dtype);  // O = sweep(q, k, v)
+    if (which == 0) return sweep_workspace_bytes(bh, n, d, e, 1, dtype, o);  // O = sweep(q, k, v)
     // dQ = sweep(dO, v, k); then dK and dV, together when d == e
-    size_t need = sweep_workspace_bytes(bh, n, e, d, 1, dtype);
-    const size_t rest = d == e ? sweep_workspace_bytes(bh, n, d, e, 2, dtype)
-                               : std::max(sweep_workspace_bytes(bh, n, e, d, 1, dtype), sweep_workspace_bytes(bh, n, d, e, 1, dtype));
+    size_t need = sweep_workspace_bytes(bh, n, e, d, 1, dtype, o);
+    const size_t rest = d == e && o.paired != LA_OPT_OFF
+                            ? sweep_workspace_bytes(bh, n, d, e, 2, dtype, o)
+                            : std::max(sweep_workspace_bytes(bh, n, e, d, 1, dtype, o), sweep_workspace_bytes(bh, n, d, e, 1, dtype, o));
     return std::max(need, rest);
+}
+
+extern "C" size_t la_workspace_bytes(int which, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype) {
+    return la_workspace_bytes_opts(which, b, h, n, d, e, dtype, nullptr);
+}
+
+extern "C" int la_fwd_opts(const void* q, const void* k, const void* v, const float* s, void* o, const int64_t* strides,
+                           int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype, void* workspace,
+                           size_t ws_bytes, const la_launch_opts* opts, void* stream) {
+    const la::Scratch ws = {workspace, workspace ? ws_bytes : 0};
+    const la::Opts& op = opts ? *opts : la::kAuto;
+    const hipStream_t st = static_cast<hipStream_t>(stream);
+    using la::dense;
+    using la::strided;
+    if (!strides)
+        return la::fwd(dense(q, h, n, d), dense(k, h, n, d), dense(v, h, n, e), s, dense(o, h, n, e), b, h, n, d, e, dtype, ws, op, st);
+    return la::fwd(strided(q, strides), strided(k, strides + 3), strided(v, strides + 6), s, strided(o, strides + 9), b, h, n,
+                   d, e, dtype, ws, op, st);
+}
+
+extern "C" int la_bwd_opts(const void* q, const void* k, const void* v, const float* s, const void* dout, void* dq,
+                           void* dk, void* dv, const int64_t* strides, int64_t b, int64_t h, int64_t n, int64_t d,
+                           int64_t e, int dtype, void* workspace, size_t ws_bytes, const la_launch_opts* opts, void* stream) {
+    const la::Scratch ws = {workspace, workspace ? ws_bytes : 0};
+    const la::Opts& op = opts ? *opts : la::kAuto;
+    const hipStream_t st = static_cast<hipStream_t>(stream);
+    using la::dense;
+    using la::strided;
+    if (!strides)
+        return la::bwd(dense(q, h, n, d), dense(k, h, n, d), dense(v, h, n, e), s, dense(dout, h, n, e), dense(dq, h, n, d),
+                       dense(dk, h, n, d), dense(dv, h, n, e), b, h, n, d, e, dtype, ws, op, st);
+    return la::bwd(strided(q, strides), strided(k, strides + 3), strided(v, strides + 6), s, strided(dout, strides + 9),
+                   strided(dq, strides + 12), strided(dk, strides + 15), strided(dv, strides + 18), b, h, n, d, e, dtype, ws,
+                   op, st);
 }
 
 extern "C" int la_fwd(const void* q, const void* k, const void* v, const float* s, void* o, int64_t b, int64_t h,
                       int64_t n, int64_t d, int64_t e, int dtype, void* workspace, size_t ws_bytes, void* stream) {
-    const la::Scratch ws = {workspace, workspace ? ws_bytes : 0};
-    using la::dense;
-    return la::fwd(dense(q, h, n, d), dense(k, h, n, d), dense(v, h, n, e), s, dense(o, h, n, e), b, h, n, d, e, dtype,
-                   ws, static_cast<hipStream_t>(stream));
+    return la_fwd_opts(q, k, v, s, o, nullptr, b, h, n, d, e, dtype, workspace, ws_bytes, nullptr, stream);
 }
 
 extern "C" int la_bwd(const void* q, const void* k, const void* v, const float* s, const void* dout, void* dq,
                       void* dk, void* dv, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
                       void* workspace, size_t ws_bytes, void* stream) {
-    const la::Scratch ws = {workspace, workspace ? ws_bytes : 0};
-    using la::dense;
-    return la::bwd(dense(q, h, n, d), dense(k, h, n, d), dense(v, h, n, e), s, dense(dout, h, n, e), dense(dq, h, n, d),
-                   dense(dk, h, n, d), dense(dv, h, n, e), b, h, n, d, e, dtype, ws, static_cast<hipStream_t>(stream));
+    return la_bwd_opts(q, k, v, s, dout, dq, dk, dv, nullptr, b, h, n, d, e, dtype, workspace, ws_bytes, nullptr, stream);
 }
 
 extern "C" int la_fwd_strided(const void* q, const void* k, const void* v, const float* s, void* o,
                               const int64_t* strides, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
                               void* workspace, size_t ws_bytes, void* stream) {
-    const la::Scratch ws = {workspace, workspace ? ws_bytes : 0};
     if (!strides) return LA_E_NULLPTR;
-    using la::strided;
-    return la::fwd(strided(q, strides), strided(k, strides + 3), strided(v, strides + 6), s, strided(o, strides + 9), b,
-                   h, n, d, e, dtype, ws, static_cast<hipStream_t>(stream));
+    return la_fwd_opts(q, k, v, s, o, strides, b, h, n, d, e, dtype, workspace, ws_bytes, nullptr, stream);
 }
 
 extern "C" int la_bwd_strided(const void* q, const void* k, const void* v, const float* s, const void* dout, void* dq,
                               void* dk, void* dv, const int64_t* strides, int64_t b, int64_t h, int64_t n, int64_t d,
                               int64_t e, int dtype, void* workspace, size_t ws_bytes, void* stream) {
-    const la::Scratch ws = {workspace, workspace ? ws_bytes : 0};
     if (!strides) return LA_E_NULLPTR;
-    using la::strided;
-    return la::bwd(strided(q, strides), strided(k, strides + 3), strided(v, strides + 6), s, strided(dout, strides + 9),
-                   strided(dq, strides + 12), strided(dk, strides + 15), strided(dv, strides + 18), b, h, n, d, e, dtype,
-                   ws, static_cast<hipStream_t>(stream));
+    return la_bwd_opts(q, k, v, s, dout, dq, dk, dv, strides, b, h, n, d, e, dtype, workspace, ws_bytes, nullptr, stream);
 }

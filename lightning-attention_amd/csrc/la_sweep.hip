@@ -23,8 +23,6 @@
 // contraction index on the B side.  Transposed operands (y^T, z^T) come from the
 // LDS transpose read ds_read_b64_tr_b16.  x/y/z tiles are double-buffered in LDS
 // (global -> registers one block ahead -> LDS), two barriers per block.
-#include <stdlib.h>
-
 #include "la_sweep_common.h"
 #include "lightning_attn_hip.h"
 
@@ -482,11 +480,8 @@ template <typename T, int DKP, bool DECAY>
 static int launch_both_one(const SweepBoth& b, hipStream_t st) {
     constexpr size_t lds = SweepLds<DKP>::bytes(sizeof(T));
     auto kern = la_sweep_both_kernel<T, DKP, DECAY>;
-    if (lds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-    }
+    static unsigned char lds_allowed[kMaxDevices];
+    if (const int e = allow_lds(kern, lds, lds_allowed)) return e;
     hipLaunchKernelGGL(kern, dim3(b.nfwd + part_grid(b.rev)), dim3(512), lds, st, b);
     return (int)hipGetLastError();
 }
@@ -507,11 +502,8 @@ static int launch_one(const SweepPair& pair, hipStream_t st) {
     constexpr size_t lds = SweepLds<DKP>::bytes(sizeof(T));
     static_assert(lds <= 160 * 1024, "LDS budget");
     auto kern = la_sweep_kernel<T, DKP, REVERSE, DECAY>;
-    if (lds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-    }
+    static unsigned char lds_allowed[kMaxDevices];
+    if (const int e = allow_lds(kern, lds, lds_allowed)) return e;
     const int units8 = (a.bh + 7) / 8 * 8;
     const unsigned grid = (unsigned)(units8 * a.nslice * a.nchunk * pair.nprod);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, st, pair);
@@ -541,7 +533,7 @@ static int num_cus() {
 // leaves most of the 256 CUs idle; the walk is then cut into up to 8 chunks whose workgroups
 // rebuild their incoming state themselves.  A warm-up block costs about half a full block, so
 // chunk lengths shrink geometrically (len_c ~ (1 - rho)^c, rho = 0.5) to make all workgroups
-// finish together.  LA_SWEEP_CHUNKS=<C> overrides the count.
+// finish together.  The caller's launch options can override the count.
 static int64_t warm_up_chunks(int64_t wgs, int64_t nblk) {
     const int64_t cus = num_cus();
     int64_t c = 1;
@@ -552,9 +544,7 @@ static int64_t warm_up_chunks(int64_t wgs, int64_t nblk) {
     return c > 8 ? 8 : c < 1 ? 1 : c;
 }
 
-void plan_warm_up_chunks(int64_t wgs, int64_t nblk, int* nchunk, int* chunk_start /* [9] */) {
-    const char* env = getenv("LA_SWEEP_CHUNKS");  // read per call so that tests can vary it
-    const int forced = env ? atoi(env) : 0;
+void plan_warm_up_chunks(int64_t wgs, int64_t nblk, int forced, int* nchunk, int* chunk_start /* [9] */) {
     int64_t c = forced > 0 ? forced : warm_up_chunks(wgs, nblk);
     if (c > 8) c = 8;
     if (c > nblk) c = nblk;
@@ -578,8 +568,8 @@ void plan_warm_up_chunks(int64_t wgs, int64_t nblk, int* nchunk, int* chunk_star
     for (int i = (int)c; i < 9; ++i) chunk_start[i] = (int)nblk;
 }
 
-static void choose_chunks(SweepArgs& a, int nprod = 1) {
-    plan_warm_up_chunks((int64_t)((a.bh + 7) / 8 * 8) * a.nslice * nprod, (a.n + 63) / 64, &a.nchunk, a.chunk_start);
+static void choose_chunks(SweepArgs& a, int nprod, const Opts& opts) {
+    plan_warm_up_chunks((int64_t)((a.bh + 7) / 8 * 8) * a.nslice * nprod, (a.n + 63) / 64, opts.chunks, &a.nchunk, a.chunk_start);
 }
 
 static SweepArgs make_args(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv) {
@@ -617,7 +607,7 @@ static int launch_classic(const SweepPair& p, int dtype, bool reverse, hipStream
 // With a workspace the kernels do not rebuild a chunk's incoming state with warm-up blocks: the states
 // the chunks end with are collected and scanned, and every chunk starts from the result (three
 // launches; equally long chunks, up to 64 of them).  Number of chunks and bytes of workspace for a
-// launch of nprod sweeps, 0 bytes where the warm-up form is used.  LA_SWEEP_SCAN=0 keeps to the warm-up form.
+// launch of nprod sweeps, 0 bytes where the warm-up form is used (always, with opts.scan == LA_OPT_OFF).
 struct ScanPlan {
     int nchunk, chunk_len;
     size_t bytes;
@@ -639,13 +629,11 @@ static double warm_up_us(int64_t bh, int64_t n, int64_t dk, int64_t dv, int npro
     return warm_up_frac(wgs, nblk) * (double)nblk * block_us(dk, wide);
 }
 
-static ScanPlan plan_scan(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, bool wide) {
+static ScanPlan plan_scan(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, bool wide, const Opts& opts) {
     const ScanPlan none = {1, 0, 0, warm_up_us(bh, n, dk, dv, nprod, wide)};
     ScanPlan pl = none;
-    const char* off = getenv("LA_SWEEP_SCAN");
-    if (off && atoi(off) == 0) return none;
-    const char* env = getenv("LA_SWEEP_CHUNKS");
-    const int forced = env ? atoi(env) : 0;
+    if (opts.scan == LA_OPT_OFF) return none;
+    const int forced = opts.chunks;
     const int64_t nblk = (n + 63) / 64, cus = num_cus();
     const int64_t nslice = wide ? 1 : (dv + 63) / 64;
     const int64_t wgs = (bh + 7) / 8 * 8 * nslice * nprod;
@@ -672,11 +660,10 @@ static ScanPlan plan_scan(int64_t bh, int64_t n, int64_t dk, int64_t dv, int npr
 // turns the saved work into time (dK + dV at the headline shape: 0.31 against 0.415 ms) - as long
 // as there are workgroups enough.  A 128-column workgroup takes about 1.25 times as long as a
 // 64-column one, and there are half as many: compare the rounds of workgroups the chip has to run.
-// `scratch`: bytes of workspace the caller has.  LA_SWEEP_WIDE=0 / 1 overrides the choice.
-static bool wide_columns(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, size_t scratch) {
+// `scratch`: bytes of workspace the caller has.  opts.wide overrides the choice.
+static bool wide_columns(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, size_t scratch, const Opts& opts) {
     if (dk > 128 || dv <= 64 || dv > 128) return false;
-    const char* env = getenv("LA_SWEEP_WIDE");
-    if (env) return atoi(env) != 0;
+    if (opts.wide != LA_OPT_AUTO) return opts.wide == LA_OPT_ON;
     if (dk <= 64) return false;  // the 128-column form pads the feature dim to 128
     const int64_t cus = num_cus(), wide = (bh + 7) / 8 * 8 * nprod, narrow = 2 * wide;
     if (narrow <= cus) {
@@ -684,28 +671,28 @@ static bool wide_columns(int64_t bh, int64_t n, int64_t dk, int64_t dv, int npro
         // into chunks from scanned states, rather half as many workgroups of 128 columns and twice the chunks
         // (b1 h32 n8192 fwd+bwd 0.28 against 0.34 ms, b1 h4 n65536 0.46 against 0.62).
         if (narrow * 2 > cus) return false;
-        const ScanPlan w = plan_scan(bh, n, dk, dv, nprod, true), nw = plan_scan(bh, n, dk, dv, nprod, false);
+        const ScanPlan w = plan_scan(bh, n, dk, dv, nprod, true, opts), nw = plan_scan(bh, n, dk, dv, nprod, false, opts);
         return w.nchunk > 1 && w.bytes <= scratch && w.us < (nw.bytes <= scratch ? nw.us : warm_up_us(bh, n, dk, dv, nprod, false));
     }
     return (wide + cus - 1) / cus * 5 < (narrow + cus - 1) / cus * 4;
 }
 
 // Workspace the kernels can use for one launch of nprod sweeps (0: none).
-size_t sweep_workspace_bytes(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int dtype) {
+size_t sweep_workspace_bytes(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int dtype, const Opts& opts) {
     if (dtype != LA_BF16 && dtype != LA_FP16) return 0;
-    return plan_scan(bh, n, dk, dv, nprod, wide_columns(bh, n, dk, dv, nprod, (size_t)-1)).bytes;
+    return plan_scan(bh, n, dk, dv, nprod, wide_columns(bh, n, dk, dv, nprod, (size_t)-1, opts), opts).bytes;
 }
 
 static int launch_planned(SweepPair& p, int64_t bh, int64_t n, int64_t dk, int64_t dv, int dtype, bool reverse, void* ws,
-                          size_t ws_bytes, hipStream_t st) {
+                          size_t ws_bytes, const Opts& opts, hipStream_t st) {
     const bool ws_ok = ws && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0;
-    p.wide = wide_columns(bh, n, dk, dv, p.nprod, ws_ok ? ws_bytes : 0) ? 1 : 0;
+    p.wide = wide_columns(bh, n, dk, dv, p.nprod, ws_ok ? ws_bytes : 0, opts) ? 1 : 0;
     p.mode = kWarmUp;
     p.chunk_len = 0;
     p.state = nullptr;
     for (int i = 0; i < p.nprod; ++i)
         if (p.wide) p.a[i].nslice = 1;
-    const ScanPlan pl = plan_scan(bh, n, dk, dv, p.nprod, p.wide != 0);
+    const ScanPlan pl = plan_scan(bh, n, dk, dv, p.nprod, p.wide != 0, opts);
     if (pl.nchunk > 1 && ws_ok && ws_bytes >= pl.bytes) {
         p.mode = kCollect;  // sweep_pipe runs the three launches
         p.chunk_len = pl.chunk_len;
@@ -715,7 +702,7 @@ static int launch_planned(SweepPair& p, int64_t bh, int64_t n, int64_t dk, int64
             for (int j = 0; j < 9; ++j) p.a[i].chunk_start[j] = 0;
         }
     } else {
-        choose_chunks(p.a[0], p.nprod);
+        choose_chunks(p.a[0], p.nprod, opts);
         for (int i = 1; i < p.nprod; ++i) {
             p.a[i].nchunk = p.a[0].nchunk;
             for (int j = 0; j < 9; ++j) p.a[i].chunk_start[j] = p.a[0].chunk_start[j];
@@ -728,41 +715,39 @@ static int launch_planned(SweepPair& p, int64_t bh, int64_t n, int64_t dk, int64
 
 // x,y: (b,h,n,dk)  z,out: (b,h,n,dv), each with its own batch / head / token strides
 int sweep(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
-          bool reverse, void* ws, size_t ws_bytes, hipStream_t st) {
+          bool reverse, void* ws, size_t ws_bytes, const Opts& opts, hipStream_t st) {
     SweepPair p;
     p.nprod = 1;
     p.a[0] = make_args(io, s, bh, h, n, dk, dv);
-    return launch_planned(p, bh, n, dk, dv, dtype, reverse, ws, ws_bytes, st);
+    return launch_planned(p, bh, n, dk, dv, dtype, reverse, ws, ws_bytes, opts, st);
 }
 
 // Two sweeps of the same shape and direction in one launch.
 int sweep2(const SweepIO& io0, const SweepIO& io1, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv,
-           int dtype, bool reverse, void* ws, size_t ws_bytes, hipStream_t st) {
-    if (getenv("LA_SWEEP_UNPAIRED")) {  // for measurements: two launches
-        const int rc = sweep(io0, s, bh, h, n, dk, dv, dtype, reverse, ws, ws_bytes, st);
-        return rc != LA_OK ? rc : sweep(io1, s, bh, h, n, dk, dv, dtype, reverse, ws, ws_bytes, st);
+           int dtype, bool reverse, void* ws, size_t ws_bytes, const Opts& opts, hipStream_t st) {
+    if (opts.paired == LA_OPT_OFF) {  // for measurements: two launches
+        const int rc = sweep(io0, s, bh, h, n, dk, dv, dtype, reverse, ws, ws_bytes, opts, st);
+        return rc != LA_OK ? rc : sweep(io1, s, bh, h, n, dk, dv, dtype, reverse, ws, ws_bytes, opts, st);
     }
     SweepPair p;
     p.nprod = 2;
     p.a[0] = make_args(io0, s, bh, h, n, dk, dv);
     p.a[1] = make_args(io1, s, bh, h, n, dk, dv);
-    return launch_planned(p, bh, n, dk, dv, dtype, reverse, ws, ws_bytes, st);
+    return launch_planned(p, bh, n, dk, dv, dtype, reverse, ws, ws_bytes, opts, st);
 }
 
 // The three sweeps of a backward pass with d == e (dQ forward; dK, dV reverse, paired) in ONE launch,
 // where that is the faster way: they fit on the chip together, so they run side by side, each cut into
 // the warm-up chunks the CUs left over allow.  Results are bit-identical to separate launches.
 // Returns LA_E_UNSUPPORTED when separate launches are to be used (they are estimated faster - scanned
-// chunk states on a long walk -, or the sweeps fill the chip anyway).  LA_SWEEP_ONCE=0 / 1: never /
-// whenever possible.
+// chunk states on a long walk -, or the sweeps fill the chip anyway).  opts.once = LA_OPT_OFF / LA_OPT_ON:
+// never / whenever possible.
 int sweep_bwd_once(const SweepIO& dq, const SweepIO& dk, const SweepIO& dv, const float* s, int64_t bh, int64_t h, int64_t n,
-                   int64_t d, int dtype, void* ws, size_t ws_bytes, hipStream_t st) {
+                   int64_t d, int dtype, void* ws, size_t ws_bytes, const Opts& opts, hipStream_t st) {
     if (dtype != LA_BF16 && dtype != LA_FP16) return LA_E_UNSUPPORTED;
-    const char* env = getenv("LA_SWEEP_ONCE");
-    const int forced = env ? (atoi(env) != 0 ? 1 : -1) : 0;
-    if (forced < 0 || getenv("LA_SWEEP_UNPAIRED")) return LA_E_UNSUPPORTED;
-    const char* wide_env = getenv("LA_SWEEP_WIDE");
-    if (forced == 0 && wide_env && atoi(wide_env) != 0) return LA_E_UNSUPPORTED;  // 128-column workgroups asked for
+    const int forced = opts.once == LA_OPT_ON ? 1 : opts.once == LA_OPT_OFF ? -1 : 0;
+    if (forced < 0 || opts.paired == LA_OPT_OFF) return LA_E_UNSUPPORTED;
+    if (forced == 0 && opts.wide == LA_OPT_ON) return LA_E_UNSUPPORTED;  // 128-column workgroups asked for
     const int64_t cus = num_cus(), nblk = (n + 63) / 64, nslice = (d + 63) / 64;
     const int64_t wgs = (bh + 7) / 8 * 8 * nslice * 3;  // one chunk each
     if (forced == 0) {
@@ -771,8 +756,8 @@ int sweep_bwd_once(const SweepIO& dq, const SweepIO& dk, const SweepIO& dv, cons
         const bool ws_ok = ws && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0;
         double separate = 0.0;
         for (int nprod = 1; nprod <= 2; ++nprod) {
-            const bool wide = wide_columns(bh, n, d, d, nprod, ws_ok ? ws_bytes : 0);
-            const ScanPlan pl = plan_scan(bh, n, d, d, nprod, wide);
+            const bool wide = wide_columns(bh, n, d, d, nprod, ws_ok ? ws_bytes : 0, opts);
+            const ScanPlan pl = plan_scan(bh, n, d, d, nprod, wide, opts);
             separate += pl.nchunk > 1 && ws_ok && ws_bytes >= pl.bytes ? pl.us : warm_up_us(bh, n, d, d, nprod, wide);
         }
         // here: the longest workgroup of 3 * wgs/3 * c warm-up chunked ones
@@ -791,7 +776,7 @@ int sweep_bwd_once(const SweepIO& dq, const SweepIO& dk, const SweepIO& dv, cons
         p->state = nullptr;
     }
     // the same chunks for every sweep: what all of them together leave room for
-    choose_chunks(b.fwd.a[0], 3);
+    choose_chunks(b.fwd.a[0], 3, opts);
     b.fwd.a[1] = b.fwd.a[0];
     for (int i = 0; i < 2; ++i) {
         b.rev.a[i].nchunk = b.fwd.a[0].nchunk;
@@ -807,20 +792,18 @@ int sweep_bwd_once(const SweepIO& dq, const SweepIO& dk, const SweepIO& dv, cons
 // d != e: both contract over e and produce d columns): one launch where they fit on the chip together
 // and separate launches are not estimated faster; LA_E_UNSUPPORTED otherwise.
 int sweep_fwd_rev_once(const SweepIO& fwd, const SweepIO& rev, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk,
-                       int64_t dv, int dtype, void* ws, size_t ws_bytes, hipStream_t st) {
+                       int64_t dv, int dtype, void* ws, size_t ws_bytes, const Opts& opts, hipStream_t st) {
     if (dtype != LA_BF16 && dtype != LA_FP16) return LA_E_UNSUPPORTED;
-    const char* env = getenv("LA_SWEEP_ONCE");
-    const int forced = env ? (atoi(env) != 0 ? 1 : -1) : 0;
-    if (forced < 0 || getenv("LA_SWEEP_UNPAIRED")) return LA_E_UNSUPPORTED;
-    const char* wide_env = getenv("LA_SWEEP_WIDE");
-    if (forced == 0 && wide_env && atoi(wide_env) != 0) return LA_E_UNSUPPORTED;
+    const int forced = opts.once == LA_OPT_ON ? 1 : opts.once == LA_OPT_OFF ? -1 : 0;
+    if (forced < 0 || opts.paired == LA_OPT_OFF) return LA_E_UNSUPPORTED;
+    if (forced == 0 && opts.wide == LA_OPT_ON) return LA_E_UNSUPPORTED;
     const int64_t cus = num_cus(), nblk = (n + 63) / 64, nslice = (dv + 63) / 64;
     const int64_t wgs = (bh + 7) / 8 * 8 * nslice * 2;
     if (forced == 0) {
         if (wgs > cus) return LA_E_UNSUPPORTED;
         const bool ws_ok = ws && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0;
-        const bool wide = wide_columns(bh, n, dk, dv, 1, ws_ok ? ws_bytes : 0);
-        const ScanPlan pl = plan_scan(bh, n, dk, dv, 1, wide);
+        const bool wide = wide_columns(bh, n, dk, dv, 1, ws_ok ? ws_bytes : 0, opts);
+        const ScanPlan pl = plan_scan(bh, n, dk, dv, 1, wide, opts);
         const double separate = 2.0 * (pl.nchunk > 1 && ws_ok && ws_bytes >= pl.bytes ? pl.us : warm_up_us(bh, n, dk, dv, 1, wide));
         if (warm_up_frac(wgs, nblk) * (double)nblk * block_us(dk, false) >= separate) return LA_E_UNSUPPORTED;
     }
@@ -828,7 +811,7 @@ int sweep_fwd_rev_once(const SweepIO& fwd, const SweepIO& rev, const float* s, i
     b.fwd.nprod = b.rev.nprod = 1;
     b.fwd.a[0] = make_args(fwd, s, bh, h, n, dk, dv);
     b.rev.a[0] = make_args(rev, s, bh, h, n, dk, dv);
-    choose_chunks(b.fwd.a[0], 2);
+    choose_chunks(b.fwd.a[0], 2, opts);
     b.rev.a[0].nchunk = b.fwd.a[0].nchunk;
     for (int j = 0; j < 9; ++j) b.rev.a[0].chunk_start[j] = b.fwd.a[0].chunk_start[j];
     for (SweepPair* p : {&b.fwd, &b.rev}) {

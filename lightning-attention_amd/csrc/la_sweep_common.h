@@ -1,8 +1,12 @@
 // Definitions shared by the sweep kernels (bf16 / fp16 MFMA paths).
 #pragma once
 #include "la_common.h"
+#include "lightning_attn_hip.h"
 
 namespace la {
+
+// How the caller wants a call mapped onto launches (all zero: the library's own choices).
+typedef la_launch_opts Opts;
 
 // Where the (batch, head, token) rows of a tensor start, in elements; the feature dim is contiguous.
 // A plain (b, h, n, d) tensor has {h*n*d, n*d, d}; a (b, n, h, d) projection output viewed as
@@ -123,8 +127,26 @@ struct SweepBoth {
 int sweep_pipe_both(const SweepBoth& b, int dtype, hipStream_t st);  // feature dim up to 128, la_sweep_pipe.hip
 
 // Count (up to 8) and first blocks, chunk_start[0 .. 8], of the warm-up chunks for a launch that would have
-// `wgs` workgroups with one chunk each, on a walk of nblk blocks; defined in la_sweep.hip.
-void plan_warm_up_chunks(int64_t wgs, int64_t nblk, int* nchunk, int* chunk_start);
+// `wgs` workgroups with one chunk each, on a walk of nblk blocks; `forced` > 0 overrides the count.
+// Defined in la_sweep.hip.
+void plan_warm_up_chunks(int64_t wgs, int64_t nblk, int forced, int* nchunk, int* chunk_start);
+
+// Raises a kernel's dynamic LDS limit above the 64 KB default, once per kernel and device (the call is
+// not free and the limit stays).  `done` is the instantiation's own flag array, one entry per device.
+constexpr int kMaxDevices = 64;
+template <typename K>
+inline int allow_lds(K kern, size_t lds, unsigned char (&done)[kMaxDevices]) {
+    if (lds <= 64 * 1024) return 0;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    const bool cached = dev >= 0 && dev < kMaxDevices;
+    if (cached && __atomic_load_n(&done[dev], __ATOMIC_ACQUIRE)) return 0;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    if (cached) __atomic_store_n(&done[dev], (unsigned char)1, __ATOMIC_RELEASE);
+    return 0;
+}
 
 // Launches the single-barrier pipelined kernel (feature dim up to 128); defined in la_sweep_pipe.hip.
 // n, dk, dv, h, bh, nslice and the chunking must agree between the two sweeps of a pair.

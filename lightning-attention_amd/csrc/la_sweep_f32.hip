@@ -282,11 +282,8 @@ template <int DKP, bool DECAY>
 static int launch_trio_f32(const SweepTrioF32& t, hipStream_t st) {
     constexpr size_t lds = (size_t)(2 * 64 * (DKP + LA_F32_XPAD) + 2 * 64 * 68) * sizeof(float);
     auto kern = la_sweep_f32_trio_kernel<DKP, DECAY>;
-    if (lds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-    }
+    static unsigned char lds_allowed[kMaxDevices];
+    if (const int e = allow_lds(kern, lds, lds_allowed)) return e;
     hipLaunchKernelGGL(kern, dim3(3 * t.per_part), dim3(256), lds, st, t);
     return (int)hipGetLastError();
 }
@@ -295,11 +292,8 @@ template <int DKP, bool REVERSE, bool DECAY>
 static int launch_one_f32(const SweepArgsF32& a, hipStream_t st) {
     constexpr size_t lds = (size_t)(2 * 64 * (DKP + LA_F32_XPAD) + 2 * 64 * 68) * sizeof(float);
     auto kern = la_sweep_f32_kernel<DKP, REVERSE, DECAY>;
-    if (lds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-    }
+    static unsigned char lds_allowed[kMaxDevices];
+    if (const int e = allow_lds(kern, lds, lds_allowed)) return e;
     const int units8 = (a.bh + 7) / 8 * 8;
     hipLaunchKernelGGL(kern, dim3((unsigned)(units8 * a.nslice * a.nchunk)), dim3(256), lds, st, a);
     return (int)hipGetLastError();
@@ -327,23 +321,23 @@ static SweepArgsF32 make_args_f32(const void* x, const void* y, const void* z, v
 }
 
 int sweep_f32(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
-              int64_t n, int64_t dk, int64_t dv, bool reverse, hipStream_t st) {
+              int64_t n, int64_t dk, int64_t dv, bool reverse, int chunks, hipStream_t st) {
     if (dk > 128) return LA_E_UNSUPPORTED;
     SweepArgsF32 a = make_args_f32(x, y, z, out, s, bh, h, n, dk, dv);
-    plan_warm_up_chunks((bh + 7) / 8 * 8 * a.nslice, (n + 63) / 64, &a.nchunk, a.chunk_start);
+    plan_warm_up_chunks((bh + 7) / 8 * 8 * a.nslice, (n + 63) / 64, chunks, &a.nchunk, a.chunk_start);
     return reverse ? launch_dir_f32<true>(a, st) : launch_dir_f32<false>(a, st);
 }
 
 // float32 backward pass with d == e: dQ = fwd(dO, v, k), dK = rev(v, dO, q), dV = rev(k, q, dO) in one
 // launch (the sweeps are independent; with few sequences they run side by side).
 int sweep_f32_bwd_once(const void* q, const void* k, const void* v, const void* dout, void* dq, void* dk, void* dv,
-                       const float* s, int64_t bh, int64_t h, int64_t n, int64_t d, hipStream_t st) {
+                       const float* s, int64_t bh, int64_t h, int64_t n, int64_t d, int chunks, hipStream_t st) {
     if (d > 128) return LA_E_UNSUPPORTED;
     SweepTrioF32 t;
     t.a[0] = make_args_f32(dout, v, k, dq, s, bh, h, n, d, d);
     t.a[1] = make_args_f32(v, dout, q, dk, s, bh, h, n, d, d);
     t.a[2] = make_args_f32(k, q, dout, dv, s, bh, h, n, d, d);
-    plan_warm_up_chunks((bh + 7) / 8 * 8 * t.a[0].nslice * 3, (n + 63) / 64, &t.a[0].nchunk, t.a[0].chunk_start);
+    plan_warm_up_chunks((bh + 7) / 8 * 8 * t.a[0].nslice * 3, (n + 63) / 64, chunks, &t.a[0].nchunk, t.a[0].chunk_start);
     for (int i = 1; i < 3; ++i) {
         t.a[i].nchunk = t.a[0].nchunk;
         for (int j = 0; j < 9; ++j) t.a[i].chunk_start[j] = t.a[0].chunk_start[j];

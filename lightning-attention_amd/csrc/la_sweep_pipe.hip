@@ -613,11 +613,8 @@ static int launch_one(const SweepPair& pair, hipStream_t st) {
     constexpr size_t lds = PipeLds<DKP, NH>::bytes(sizeof(T));
     static_assert(lds <= 160 * 1024, "LDS budget");
     auto kern = la_sweep_pipe_kernel<T, DKP, NH, REVERSE, DECAY, DENSE>;
-    if (lds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-    }
+    static unsigned char lds_allowed[kMaxDevices];
+    if (const int e = allow_lds(kern, lds, lds_allowed)) return e;
     const int units8 = (a.bh + 7) / 8 * 8;
     // the state slots the host sized must be the ones this instantiation reads and writes
     if (pair.mode != kWarmUp && pipe_state_floats(a.dk, pair.wide != 0) != (size_t)4 * NH * (DKP / 16) * 64 * 4) return LA_E_WORKSPACE;
@@ -657,11 +654,8 @@ template <typename T, int DKP, bool DECAY, bool DENSE>
 static int launch_both_one(const SweepBoth& b, hipStream_t st) {
     constexpr size_t lds = PipeLds<DKP, 1>::bytes(sizeof(T));
     auto kern = la_sweep_pipe_both_kernel<T, DKP, DECAY, DENSE>;
-    if (lds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-    }
+    static unsigned char lds_allowed[kMaxDevices];
+    if (const int e = allow_lds(kern, lds, lds_allowed)) return e;
     hipLaunchKernelGGL(kern, dim3(b.nfwd + part_grid(b.rev)), dim3(512), lds, st, b);
     return (int)hipGetLastError();
 }

@@ -6,3 +6,4 @@ from .lightning_attn2 import (  # noqa: F401
     lightning_attn2_parallel,
 )
 from .srmsnorm import SimpleRMSNorm, _SrmsNorm  # noqa: F401
+from ._lib import launch_opts  # noqa: F401

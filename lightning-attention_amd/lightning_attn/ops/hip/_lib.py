@@ -2,6 +2,7 @@
 
 The library is loaded on first use.  A missing library is a hard error: there is
 no CPU or eager fallback behind these operators."""
+import contextlib
 import ctypes
 import os
 import threading
@@ -16,13 +17,51 @@ _DTYPES = {torch.bfloat16: LA_BF16, torch.float16: LA_FP16, torch.float32: LA_FP
 
 SYMBOLS = (
     "la_version", "la_error_string", "la_supported", "la_workspace_bytes",
-    "la_fwd", "la_bwd", "la_fwd_strided", "la_bwd_strided", "srmsnorm_fwd", "srmsnorm_bwd",
+    "la_fwd", "la_bwd", "la_fwd_strided", "la_bwd_strided", "la_workspace_bytes_opts", "la_fwd_opts", "la_bwd_opts",
+    "srmsnorm_fwd", "srmsnorm_bwd",
 )
 
 _lib = None
 _lock = threading.Lock()
 
 _vp, _i64, _int, _sz, _f = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t, ctypes.c_float
+
+LA_OPT_AUTO, LA_OPT_OFF, LA_OPT_ON = 0, 1, 2
+
+
+class LaunchOpts(ctypes.Structure):
+    """la_launch_opts of the header: all zero = the library's own choices."""
+    _fields_ = [("chunks", ctypes.c_int32), ("scan", ctypes.c_int32), ("wide", ctypes.c_int32),
+                ("paired", ctypes.c_int32), ("once", ctypes.c_int32)]
+
+    def key(self):
+        return (self.chunks, self.scan, self.wide, self.paired, self.once)
+
+
+_tls = threading.local()
+
+
+def current_opts():
+    """The launch options in force on this thread (None: the library's own choices)."""
+    return getattr(_tls, "opts", None)
+
+
+def _tri(v):
+    return LA_OPT_AUTO if v is None else (LA_OPT_ON if v else LA_OPT_OFF)
+
+
+@contextlib.contextmanager
+def launch_opts(chunks=0, scan=None, wide=None, paired=None, once=None):
+    """Within the block, the attention operators called from this thread map their work onto
+    launches as told (the backward pass of an operator follows the options its forward ran under): `chunks` sequence chunks (0 = library's choice); `scan`, `wide`, `paired`,
+    `once` = None (library's choice) / False / True.  For measurements and tests; the results do
+    not depend on it beyond rounding (see la_launch_opts in the header)."""
+    prev = current_opts()
+    _tls.opts = LaunchOpts(int(chunks or 0), _tri(scan), _tri(wide), _tri(paired), _tri(once))
+    try:
+        yield _tls.opts
+    finally:
+        _tls.opts = prev
 
 
 def lib():
@@ -55,6 +94,14 @@ def lib():
             L.la_bwd_strided.restype = _int
             L.la_bwd_strided.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
                                          _int, _vp, _sz, _vp]
+            _op = ctypes.POINTER(LaunchOpts)
+            L.la_workspace_bytes_opts.restype = _sz
+            L.la_workspace_bytes_opts.argtypes = [_int, _i64, _i64, _i64, _i64, _i64, _int, _op]
+            L.la_fwd_opts.restype = _int
+            L.la_fwd_opts.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _sz, _op, _vp]
+            L.la_bwd_opts.restype = _int
+            L.la_bwd_opts.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
+                                      _vp, _sz, _op, _vp]
             L.srmsnorm_fwd.restype = _int
             L.srmsnorm_fwd.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _f, _int, _vp]
             L.srmsnorm_bwd.restype = _int
@@ -81,6 +128,33 @@ def require_gpu(t, what):
             "%s runs only on a HIP device: got a %s tensor (there is no CPU fallback; "
             "use lightning_attn.ops.linear_attn / SimpleRMSNormTorch for plain PyTorch)" % (what, t.device)
         )
+
+
+def require_same_device(what, **tensors):
+    """Every tensor whose pointer goes to a kernel must live on one HIP device: a host pointer, or
+    one of another GPU, handed to a launch is a memory fault, not a Python error."""
+    it = iter(tensors.items())
+    name0, t0 = next(it)
+    require_gpu(t0, what)
+    for name, t in it:
+        if t.device != t0.device:
+            raise RuntimeError("%s: %s is on %s but %s is on %s; all tensors must be on the same HIP device"
+                               % (what, name, t.device, name0, t0.device))
+
+
+_ws_cache = {}
+
+
+def workspace_bytes(which, b, h, n, d, e, code, opts):
+    """la_workspace_bytes_opts, remembered per shape: the answer depends on the arguments alone."""
+    key = (which, b, h, n, d, e, code, opts.key() if opts is not None else None, torch.cuda.current_device())
+    got = _ws_cache.get(key)
+    if got is None:
+        got = lib().la_workspace_bytes_opts(which, b, h, n, d, e, code, ctypes.byref(opts) if opts is not None else None)
+        if len(_ws_cache) > 4096:
+            _ws_cache.clear()
+        _ws_cache[key] = got
+    return got
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)

@@ -56,7 +56,7 @@ def _strides(*tensors):
 
 
 def _fwd(q, k, v, s):
-    _lib.require_gpu(q, "lightning_attn2")
+    _lib.require_same_device("lightning_attn2", q=q, k=k, v=v)
     if not (q.dtype == k.dtype == v.dtype):
         raise TypeError("q, k, v must share a dtype")
     if q.dim() != 4 or k.shape != q.shape or v.dim() != 4 or v.shape[:3] != q.shape[:3]:
@@ -72,42 +72,40 @@ def _fwd(q, k, v, s):
     L = _lib.lib()
     code = _lib.dtype_code(q.dtype)
     o = torch.empty_like(v)  # same sizes as v; dense, in v's memory order
-    ws_bytes = L.la_workspace_bytes(0, b, h, n, d, e, code)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
-    sp = s.data_ptr() if s is not None else None
-    wp = ws.data_ptr() if ws is not None else None
+    opts = _lib.current_opts()
     with _lib.on_device(q.device):
-        if all(t.is_contiguous() for t in (q, k, v, o)):
-            rc = L.la_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, o.data_ptr(), b, h, n, d, e, code, wp, ws_bytes,
-                          _lib.stream_ptr(q.device))
-        else:
-            rc = L.la_fwd_strided(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, o.data_ptr(), _strides(q, k, v, o),
-                                  b, h, n, d, e, code, wp, ws_bytes, _lib.stream_ptr(q.device))
+        ws_bytes = _lib.workspace_bytes(0, b, h, n, d, e, code, opts)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
+        sp = s.data_ptr() if s is not None else None
+        wp = ws.data_ptr() if ws is not None else None
+        strides = None if all(t.is_contiguous() for t in (q, k, v, o)) else _strides(q, k, v, o)
+        rc = L.la_fwd_opts(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, o.data_ptr(), strides, b, h, n, d, e, code,
+                           wp, ws_bytes, ctypes.byref(opts) if opts is not None else None, _lib.stream_ptr(q.device))
     _lib.check(rc, "la_fwd")
     return o, q, k, v, s
 
 
-def _bwd(q, k, v, s, do):
+def _bwd(q, k, v, s, do, opts=None):
     b, h, n, d = q.shape
     e = v.shape[-1]
     L = _lib.lib()
     code = _lib.dtype_code(q.dtype)
+    if do.device != q.device:
+        raise RuntimeError("lightning_attn2 backward: the upstream gradient is on %s, the inputs on %s" % (do.device, q.device))
     if do.dtype != q.dtype:
         do = do.to(q.dtype)
     do = _usable(do)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    ws_bytes = L.la_workspace_bytes(1, b, h, n, d, e, code)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
-    sp = s.data_ptr() if s is not None else None
-    wp = ws.data_ptr() if ws is not None else None
     with _lib.on_device(q.device):
-        if all(t.is_contiguous() for t in (q, k, v, do, dq, dk, dv)):
-            rc = L.la_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, do.data_ptr(), dq.data_ptr(), dk.data_ptr(),
-                          dv.data_ptr(), b, h, n, d, e, code, wp, ws_bytes, _lib.stream_ptr(q.device))
-        else:
-            rc = L.la_bwd_strided(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, do.data_ptr(), dq.data_ptr(),
-                                  dk.data_ptr(), dv.data_ptr(), _strides(q, k, v, do, dq, dk, dv), b, h, n, d, e, code,
-                                  wp, ws_bytes, _lib.stream_ptr(q.device))
+        ws_bytes = _lib.workspace_bytes(1, b, h, n, d, e, code, opts)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
+        sp = s.data_ptr() if s is not None else None
+        wp = ws.data_ptr() if ws is not None else None
+        dense = all(t.is_contiguous() for t in (q, k, v, do, dq, dk, dv))
+        strides = None if dense else _strides(q, k, v, do, dq, dk, dv)
+        rc = L.la_bwd_opts(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, do.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                           dv.data_ptr(), strides, b, h, n, d, e, code, wp, ws_bytes,
+                           ctypes.byref(opts) if opts is not None else None, _lib.stream_ptr(q.device))
     _lib.check(rc, "la_bwd")
     return dq, dk, dv
 
@@ -121,12 +119,14 @@ class LightningAttention2(torch.autograd.Function):
             raise ValueError("lightning_attn2 needs decay rates s; use lightning_attn2_no_decay")
         o, q, k, v, s = _fwd(q, k, v, s)
         ctx.save_for_backward(q, k, v, s)
+        # autograd runs backward on a thread of its own: the launch options in force now go with the node
+        ctx.la_opts = _lib.current_opts()
         return o
 
     @staticmethod
     def backward(ctx, do):
         q, k, v, s = ctx.saved_tensors
-        dq, dk, dv = _bwd(q, k, v, s, do)
+        dq, dk, dv = _bwd(q, k, v, s, do, ctx.la_opts)
         return dq, dk, dv, None
 
 
@@ -137,12 +137,13 @@ class LightningAttention2NoDecay(torch.autograd.Function):
     def forward(ctx, q, k, v):
         o, q, k, v, _ = _fwd(q, k, v, None)
         ctx.save_for_backward(q, k, v)
+        ctx.la_opts = _lib.current_opts()
         return o
 
     @staticmethod
     def backward(ctx, do):
         q, k, v = ctx.saved_tensors
-        return _bwd(q, k, v, None, do)
+        return _bwd(q, k, v, None, do, ctx.la_opts)
 
 
 lightning_attn2 = LightningAttention2.apply

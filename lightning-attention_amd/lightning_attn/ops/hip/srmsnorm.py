@@ -23,7 +23,8 @@ class _SrmsNorm(torch.autograd.Function):
         rstd = torch.empty((rows,), dtype=torch.float32, device=x.device)
         L = _lib.lib()
         with _lib.on_device(x.device):
-            rc = L.srmsnorm_fwd(x_arg.data_ptr(), y.data_ptr(), rstd.data_ptr(), rows, cols, x_arg.stride(0) if rows else cols,
+            # (torch reports an arbitrary stride for a dim of size <= 1)
+            rc = L.srmsnorm_fwd(x_arg.data_ptr(), y.data_ptr(), rstd.data_ptr(), rows, cols, x_arg.stride(0) if rows > 1 else cols,
                                 float(eps), _lib.dtype_code(x.dtype), _lib.stream_ptr(x.device))
         _lib.check(rc, "srmsnorm_fwd")
         ctx.save_for_backward(x, rstd)
@@ -36,6 +37,8 @@ class _SrmsNorm(torch.autograd.Function):
         if not x_arg.is_contiguous():
             x_arg = x_arg.contiguous()
         rows, cols = x_arg.shape
+        if dy.device != x.device:
+            raise RuntimeError("SimpleRMSNorm backward: the upstream gradient is on %s, x on %s" % (dy.device, x.device))
         dy = dy.contiguous()
         if dy.dtype != x.dtype:
             dy = dy.to(x.dtype)
@@ -46,7 +49,7 @@ class _SrmsNorm(torch.autograd.Function):
         L = _lib.lib()
         with _lib.on_device(x.device):
             rc = L.srmsnorm_bwd(x_arg.data_ptr(), dy.data_ptr(), rstd.data_ptr(), dx.data_ptr(), rows, cols,
-                                x_arg.stride(0) if rows else cols, _lib.dtype_code(x.dtype), _lib.stream_ptr(x.device))
+                                x_arg.stride(0) if rows > 1 else cols, _lib.dtype_code(x.dtype), _lib.stream_ptr(x.device))
         _lib.check(rc, "srmsnorm_bwd")
         return dx.reshape(dy.shape), None
 

@@ -13,12 +13,12 @@ sys.path.insert(0, os.path.join(ROOT, "lightning-attention_amd"))
 sys.path.insert(0, ROOT)
 
 from lightning_attn.ops import lightning_attn_func  # noqa: E402
+from lightning_attn.ops.hip import launch_opts  # noqa: E402
 from lightning_attn.utils import _build_slope_tensor  # noqa: E402
 from oracle import linear_attn_oracle as oracle  # noqa: E402
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
-KNOBS = ("LA_SWEEP_WIDE", "LA_SWEEP_CHUNKS", "LA_SWEEP_UNPAIRED", "LA_SWEEP_SCAN", "LA_SWEEP_ONCE")
 
 
 def _rel(a, r):
@@ -26,7 +26,7 @@ def _rel(a, r):
 
 
 @pytest.mark.parametrize("seed", [101, 202, 303, 404, 505])
-def test_random_cases_match_the_oracle(seed, monkeypatch):
+def test_random_cases_match_the_oracle(seed):
     rnd = random.Random(seed)
     for case in range(20):
         b, h = rnd.randint(1, 3), rnd.randint(1, 9)
@@ -38,21 +38,17 @@ def test_random_cases_match_the_oracle(seed, monkeypatch):
             d, e = min(d, 8 * rnd.randint(1, 16)), min(e, 8 * rnd.randint(1, 16))
         decay = rnd.random() < 0.75
         token_major = rnd.random() < 0.4
-        env = {}
+        env = {}  # launch options of this case
         if rnd.random() < 0.6:
-            env["LA_SWEEP_WIDE"] = rnd.choice(["0", "1"])
+            env["wide"] = rnd.choice([False, True])
         if rnd.random() < 0.6:
-            env["LA_SWEEP_CHUNKS"] = str(rnd.choice([1, 2, 3, 4, 5, 9, 17, 40, 64]))
+            env["chunks"] = rnd.choice([1, 2, 3, 4, 5, 9, 17, 40, 64])
         if rnd.random() < 0.3:
-            env["LA_SWEEP_SCAN"] = "0"
+            env["scan"] = False
         if rnd.random() < 0.2:
-            env["LA_SWEEP_UNPAIRED"] = "1"
+            env["paired"] = False
         if rnd.random() < 0.5:
-            env["LA_SWEEP_ONCE"] = rnd.choice(["0", "1"])
-        for name in KNOBS:
-            monkeypatch.delenv(name, raising=False)
-        for name, value in env.items():
-            monkeypatch.setenv(name, value)
+            env["once"] = rnd.choice([False, True])
         g = torch.Generator().manual_seed(1000 * seed + case)
 
         def make(cols, scale):
@@ -64,13 +60,12 @@ def test_random_cases_match_the_oracle(seed, monkeypatch):
         what = (seed, case, (b, h, n, d, e), dtype, decay, token_major, env)
         print(what, flush=True)  # names the case should a launch go wrong
         qg, kg, vg = (t.detach().requires_grad_() for t in (q, k, v))
-        o = lightning_attn_func(qg, kg, vg, None if s is None else s.to(DEV))
-        o.backward(do)
+        with launch_opts(**env):
+            o = lightning_attn_func(qg, kg, vg, None if s is None else s.to(DEV))
+            o.backward(do)
         torch.cuda.synchronize()
         want = oracle.linear_attn_fwd_bwd(q.cpu(), k.cpu(), v.cpu(), s, do.cpu(),
                                           torch.float64 if dtype == torch.float32 else torch.float32)
         limit = {torch.bfloat16: 1e-2, torch.float16: 2e-3, torch.float32: 1e-4}[dtype]
         for name, a, r in zip(("o", "dq", "dk", "dv"), (o.detach(), qg.grad, kg.grad, vg.grad), want):
             assert a.dtype == dtype and _rel(a, r) < limit, (what, name, _rel(a, r))
-    for name in KNOBS:
-        monkeypatch.delenv(name, raising=False)

@@ -118,3 +118,20 @@ def test_fp16_eps_clamp():
     y, _ = _run(x, torch.ones_like(x), eps=1e-9)
     want = oracle.srmsnorm(x, 1.6e-5)
     assert_close(y, want, atol=1e-3, rtol=1e-2)
+
+
+@pytest.mark.parametrize("cols, stride", [(1024, 0), (1000, 0), (1024, 7)])
+def test_single_row_with_arbitrary_stride(cols, stride):
+    """One row: the stride of a dim of size 1 is never used for addressing and may be anything (0 for
+    some expanded vectors); it must not reach the kernels as a row stride."""
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(cols, generator=g).bfloat16()
+    dy = torch.randn(1, cols, generator=g).bfloat16()
+    xd = x.to(DEV).as_strided((1, cols), (stride, 1)).requires_grad_()
+    assert xd.stride(0) == stride
+    y = SimpleRMSNorm(cols)(xd)
+    y.backward(dy.to(DEV))
+    torch.cuda.synchronize()
+    y_ref, dx_ref = oracle.srmsnorm_fwd_bwd(x.reshape(1, cols), dy, 1e-6)
+    assert_close(y.cpu(), y_ref, atol=ATOL, rtol=RTOL)
+    assert_close(xd.grad.cpu(), dx_ref, atol=ATOL, rtol=RTOL)

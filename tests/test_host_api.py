@@ -83,14 +83,12 @@ def test_host_only_entry_points():
     assert L.srmsnorm_bwd(p16, p16, p16, p16, 0, 64, 64, 0, None) == 0
 
 
-def test_workspace_query_is_consistent(monkeypatch):
+def test_workspace_query_is_consistent():
     """Properties of the scratch size over a grid of shapes (host logic only; without a device the library
     plans for 256 CUs): a whole number of state slots, never more than 63 of them per sequence, sweep and
     column slice, nothing for float32 or when the sequences fill the chip by themselves, nothing when
     scanned chunk states are switched off, and the backward pass never asks for less than the forward."""
     L = _lib.lib()
-    for name in ("LA_SWEEP_WIDE", "LA_SWEEP_CHUNKS", "LA_SWEEP_SCAN", "LA_SWEEP_UNPAIRED", "LA_SWEEP_ONCE"):
-        monkeypatch.delenv(name, raising=False)
     seen_some = False
     for b, h in ((1, 1), (1, 8), (2, 12), (1, 32), (4, 32), (8, 64)):
         for n in (64, 1000, 4096, 65536):
@@ -108,9 +106,58 @@ def test_workspace_query_is_consistent(monkeypatch):
                     seen_some = seen_some or fwd > 0
     assert seen_some
     assert L.la_workspace_bytes(0, 1, 8, 65536, 128, 128, 0) > 0
-    monkeypatch.setenv("LA_SWEEP_SCAN", "0")
-    assert L.la_workspace_bytes(0, 1, 8, 65536, 128, 128, 0) == 0
-    assert L.la_workspace_bytes(1, 1, 8, 65536, 192, 192, 0) == 0
+    no_scan = _lib.LaunchOpts(0, _lib.LA_OPT_OFF, 0, 0, 0)
+    assert L.la_workspace_bytes_opts(0, 1, 8, 65536, 128, 128, 0, ctypes.byref(no_scan)) == 0
+    assert L.la_workspace_bytes_opts(1, 1, 8, 65536, 192, 192, 0, ctypes.byref(no_scan)) == 0
+    # NULL options = the plain query; a forced chunk count sizes the workspace for that count
+    assert L.la_workspace_bytes_opts(0, 1, 8, 65536, 128, 128, 0, None) == L.la_workspace_bytes(0, 1, 8, 65536, 128, 128, 0)
+    forced = _lib.LaunchOpts(5, 0, _lib.LA_OPT_OFF, 0, 0)
+    assert L.la_workspace_bytes_opts(0, 4, 32, 8192, 128, 128, 0, ctypes.byref(forced)) == 128 * 2 * 4 * 128 * 64 * 4
+    # shapes the entry points reject need no workspace; neither do malformed options
+    assert L.la_workspace_bytes(0, 1, 8, 1 << 22, 128, 128, 0) == 0
+    assert L.la_workspace_bytes(0, 1, 8, 8192, 100, 128, 0) == 0
+    bad = _lib.LaunchOpts(0, 7, 0, 0, 0)
+    assert L.la_workspace_bytes_opts(0, 1, 8, 65536, 128, 128, 0, ctypes.byref(bad)) == 0
+
+
+def test_launch_options():
+    """la_launch_opts is validated on the host before anything is launched, and the Python context
+    that carries it restores the previous options on exit (also when nested)."""
+    L = _lib.lib()
+    buf = ctypes.create_string_buffer(64)
+    p16 = (ctypes.addressof(buf) + 15) & ~15
+    bad = _lib.LaunchOpts(0, 0, 5, 0, 0)
+    assert L.la_fwd_opts(p16, p16, p16, None, p16, None, 1, 1, 64, 64, 64, 0, None, 0, ctypes.byref(bad), None) == -2
+    neg = _lib.LaunchOpts(-1, 0, 0, 0, 0)
+    assert L.la_bwd_opts(p16, p16, p16, None, p16, p16, p16, p16, None, 1, 1, 64, 64, 64, 0, None, 0, ctypes.byref(neg), None) == -2
+    assert L.la_fwd_opts(None, p16, p16, None, p16, None, 1, 1, 64, 64, 64, 0, None, 0, None, None) == -1
+    from lightning_attn.ops.hip import launch_opts
+    assert _lib.current_opts() is None
+    with launch_opts(chunks=3, wide=True) as outer:
+        assert outer.key() == (3, 0, 2, 0, 0) and _lib.current_opts() is outer
+        with launch_opts(scan=False, paired=False, once=True) as inner:
+            assert inner.key() == (0, 1, 0, 1, 2) and _lib.current_opts() is inner
+        assert _lib.current_opts() is outer
+    assert _lib.current_opts() is None
+
+
+class _FakeTensor:
+    def __init__(self, device):
+        self.device = torch.device(device)
+        self.is_cuda = self.device.type == "cuda"
+
+
+def test_tensors_must_share_a_device():
+    """A host pointer (or one of another GPU) must never reach a launch: the check that stops it
+    runs on the host, so stand-in objects with a device are enough to exercise it."""
+    ok = _FakeTensor("cuda:0")
+    _lib.require_same_device("op", q=ok, k=_FakeTensor("cuda:0"), v=ok)
+    with pytest.raises(RuntimeError, match="same HIP device"):
+        _lib.require_same_device("op", q=ok, k=_FakeTensor("cpu"), v=ok)
+    with pytest.raises(RuntimeError, match="same HIP device"):
+        _lib.require_same_device("op", q=ok, k=ok, v=_FakeTensor("cuda:1"))
+    with pytest.raises(RuntimeError, match="HIP device"):
+        _lib.require_same_device("op", q=_FakeTensor("cpu"), k=ok, v=ok)
 
 
 def test_no_cpu_fallback():
