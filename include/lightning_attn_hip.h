@@ -144,6 +144,25 @@ int la_bwd_opts(const void *q, const void *k, const void *v, const float *s, con
                 void *workspace, size_t ws_bytes, const la_launch_opts *opts, void *stream);
 
 /*
+ * la_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc) and so cannot supply the workspace that makes few
+ * long sequences fast: same arguments without the workspace pair, same results bit for bit as la_fwd
+ * given la_workspace_bytes(0, ...) bytes.  The chunk states go into a static device array of
+ * LA_STATIC_SCRATCH_BYTES inside the library, which every GPU the library runs on holds until the
+ * process ends.  The call allocates and frees nothing.  Shapes whose plan needs more than the array
+ * holds are rejected with LA_E_WORKSPACE before anything is launched (the plans the library makes for
+ * a chip of up to 256 compute units always fit).  All calls on one GPU share the array: calls that
+ * follow each other on one stream are safe, calls that overlap on one GPU (different streams or
+ * threads) race on it.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress); make it outside graph capture.
+ * No counterpart in the reference (its operators allocate through torch,
+ * lightning_attn/ops/triton/lightning_attn2.py:408).
+ */
+#define LA_STATIC_SCRATCH_BYTES (16u << 20)
+int la_fwd_static(const void *q, const void *k, const void *v, const float *s, void *o,
+                  int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype, void *stream);
+
+/*
  * SimpleRMSNorm forward: rstd[r] = 1/sqrt(mean(x[r,:]^2) + eps), y = x * rstd.
  * x,y: rows x cols with `row_stride` elements between rows; rstd: rows floats.
  * Replaces _SrmsNorm.forward + srms_norm_fw

@@ -230,6 +230,49 @@ extern "C" int la_bwd(const void* q, const void* k, const void* v, const float* 
     return la_bwd_opts(q, k, v, s, dout, dq, dk, dv, nullptr, b, h, n, d, e, dtype, workspace, ws_bytes, nullptr, stream);
 }
 
+// ---- forward without any allocation: the chunk states live in a static device array ----------------
+// Each GPU the library runs on holds its own copy of the array, at its own address, until the process
+// ends.  In host code the array's name is only a handle: the address kernels can use comes from
+// hipGetSymbolAddress, asked once per device with that device current, and is kept per device.
+namespace la {
+static __device__ __align__(256) unsigned char scratch[LA_STATIC_SCRATCH_BYTES];
+static void* scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device.
+static int static_scratch(void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return LA_E_UNSUPPORTED;
+    void* p = __atomic_load_n(&scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (!p) {
+        // (two threads arriving together both ask and both get the same answer)
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return (int)hipErrorInvalidSymbol;
+        __atomic_store_n(&scratch_ptr[dev], p, __ATOMIC_RELEASE);
+    }
+    *out = p;
+    return LA_OK;
+}
+}  // namespace la
+
+extern "C" int la_fwd_static(const void* q, const void* k, const void* v, const float* s, void* o, int64_t b, int64_t h,
+                             int64_t n, int64_t d, int64_t e, int dtype, void* stream) {
+    // what la_fwd would use of a caller's workspace for this shape; host arithmetic only
+    const size_t need = la_workspace_bytes(0, b, h, n, d, e, dtype);
+    if (need > (size_t)LA_STATIC_SCRATCH_BYTES) return LA_E_WORKSPACE;
+    void* ws = nullptr;
+    if (need > 0) {
+        const int rc = la::static_scratch(&ws);
+        if (rc != LA_OK) return rc;
+    }
+    // Every state slot the scan reads is written by the collect launch before it (state waves without
+    // live columns write zeros), so nothing in the array has to start at zero and what an earlier call
+    // left there does not matter.
+    return la_fwd(q, k, v, s, o, b, h, n, d, e, dtype, ws, need, stream);
+}
+
 extern "C" int la_fwd_strided(const void* q, const void* k, const void* v, const float* s, void* o,
                               const int64_t* strides, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
                               void* workspace, size_t ws_bytes, void* stream) {

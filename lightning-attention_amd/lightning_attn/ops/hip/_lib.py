@@ -18,6 +18,7 @@ _DTYPES = {torch.bfloat16: LA_BF16, torch.float16: LA_FP16, torch.float32: LA_FP
 SYMBOLS = (
     "la_version", "la_error_string", "la_supported", "la_workspace_bytes",
     "la_fwd", "la_bwd", "la_fwd_strided", "la_bwd_strided", "la_workspace_bytes_opts", "la_fwd_opts", "la_bwd_opts",
+    "la_fwd_static",
     "srmsnorm_fwd", "srmsnorm_bwd",
 )
 
@@ -102,6 +103,8 @@ def lib():
             L.la_bwd_opts.restype = _int
             L.la_bwd_opts.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
                                       _vp, _sz, _op, _vp]
+            L.la_fwd_static.restype = _int
+            L.la_fwd_static.argtypes = [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp]
             L.srmsnorm_fwd.restype = _int
             L.srmsnorm_fwd.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _f, _int, _vp]
             L.srmsnorm_bwd.restype = _int

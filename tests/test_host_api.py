@@ -120,6 +120,31 @@ def test_workspace_query_is_consistent():
     assert L.la_workspace_bytes_opts(0, 1, 8, 65536, 128, 128, 0, ctypes.byref(bad)) == 0
 
 
+def test_static_scratch_holds_every_plan_of_the_forward():
+    """la_fwd_static rejects shapes whose plan needs more than its static array (LA_E_WORKSPACE): over a
+    grid of shapes, on a chip of 256 compute units (what the library plans for without a device), no
+    forward plan does, so nothing that la_fwd accepts is turned away there."""
+    L = _lib.lib()
+    text = open(HEADER).read()
+    cap = re.search(r"#define LA_STATIC_SCRATCH_BYTES \((\d+)u << (\d+)\)", text)
+    cap = int(cap.group(1)) << int(cap.group(2))
+    assert cap == 16 << 20
+    worst = 0
+    for b, h in ((1, 1), (1, 2), (1, 3), (1, 4), (1, 8), (2, 12), (1, 16), (1, 32), (3, 5), (1, 64), (1, 120)):
+        for n in (1000, 4096, 8192, 65536, 1 << 20):
+            for d in (64, 128, 192, 256):
+                for e in (64, 128, 192, 256):
+                    worst = max(worst, L.la_workspace_bytes(0, b, h, n, d, e, 0))
+    assert 0 < worst <= cap
+    assert b"workspace" in L.la_error_string(-4)
+    # its argument checks are la_fwd's and run before the device is touched
+    buf = ctypes.create_string_buffer(64)
+    p16 = (ctypes.addressof(buf) + 15) & ~15
+    assert L.la_fwd_static(None, p16, p16, None, p16, 1, 1, 64, 64, 64, 0, None) == -1
+    assert L.la_fwd_static(p16, p16, p16, None, p16, 1, 1, 64, 100, 64, 0, None) == -3
+    assert L.la_fwd_static(p16, p16, p16, None, p16, 0, 1, 64, 64, 64, 0, None) == 0
+
+
 def test_launch_options():
     """la_launch_opts is validated on the host before anything is launched, and the Python context
     that carries it restores the previous options on exit (also when nested)."""
