@@ -181,6 +181,30 @@ int srmsnorm_fwd(const void *x, void *y, float *rstd, int64_t rows, int64_t cols
 int srmsnorm_bwd(const void *x, const void *dy, const float *rstd, void *dx,
                  int64_t rows, int64_t cols, int64_t row_stride, int dtype, void *stream);
 
+/*
+ * Gated output norm of the TNL attention block, the caller of the attention operator:
+ *     y = LayerNorm(o; weight, bias, eps) * sigmoid(g)        o, g, y: rows x cols, dense
+ * with weight, bias of cols elements in the tensors' dtype and mean, rstd (rows floats) kept for the
+ * backward pass.  One pass over o and g instead of the three PyTorch operators of
+ * examples/module/tnl_attn.py:66-69 (`self.norm(output)`, `F.sigmoid(...)`, `output * output_gate`).
+ * cols must be a multiple of 8 (4 for float32) and at most 8192 (4096): norm_gate_supported().
+ */
+int norm_gate_supported(int64_t cols, int dtype);
+int norm_gate_fwd(const void *o, const void *g, const void *weight, const void *bias, void *y,
+                  float *mean, float *rstd, int64_t rows, int64_t cols, float eps, int dtype, void *stream);
+/*
+ * Its backward pass: given dy writes d_o and d_g (rows x cols) and the column sums dweight, dbias
+ * (cols elements, tensor dtype; accumulated in float32 in a fixed order, so results are
+ * deterministic).  The partial column sums pass through `workspace`, which must hold
+ * norm_gate_workspace_bytes(rows, cols, dtype) bytes (LA_E_WORKSPACE otherwise); its contents need
+ * not survive the call.  Replaces the autograd chain of the same three operators.
+ */
+size_t norm_gate_workspace_bytes(int64_t rows, int64_t cols, int dtype);
+int norm_gate_bwd(const void *o, const void *g, const void *weight, const void *bias,
+                  const float *mean, const float *rstd, const void *dy,
+                  void *d_o, void *d_g, void *dweight, void *dbias,
+                  void *workspace, size_t ws_bytes, int64_t rows, int64_t cols, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,106 @@
+"""Condenses rocprofv3 output of a short bench.py run into the figures the bench line and the
+profile notes quote: average launch durations of the attention and norm kernels, and their HBM
+traffic per launch from the FETCH_SIZE / WRITE_SIZE counters.
+
+    cd /tmp && export TMPDIR=/tmp
+    rocprofv3 --kernel-trace --stats --output-format csv -d OUT/kt -o p -- python3 REPO/bench.py --no-cpu --no-sweep --steps 20 --warmup 5
+    rocprofv3 --pmc FETCH_SIZE --kernel-trace --output-format csv -d OUT/fetch -o p -- python3 REPO/bench.py --no-cpu --no-sweep --steps 5 --warmup 2
+    rocprofv3 --pmc WRITE_SIZE --kernel-trace --output-format csv -d OUT/write -o p -- python3 REPO/bench.py --no-cpu --no-sweep --steps 5 --warmup 2
+    python3 REPO/lightning-attention_amd/benchmarks/profile_summary.py --kt OUT/kt --fetch OUT/fetch --write OUT/write \
+        --out REPO/profiles/la_step_b4_h32_n8192_d128_bf16.counters.json
+
+Both counters report KiB per dispatch.  They are scaled by what they read for a kernel of known
+size in the same run: PyTorch's float32 -> bfloat16 cast of a [4, 32, 8192, 128] tensor (bench.py
+makes its inputs that way), which reads 512 MiB and writes 256 MiB.
+"""
+import argparse
+import collections
+import csv
+import glob
+import json
+import os
+import re
+import statistics
+
+CAST_READ = 4 * 32 * 8192 * 128 * 4
+CAST_WRITE = 4 * 32 * 8192 * 128 * 2
+
+
+def classify(name):
+    """Short key of a kernel this repository launches (or of the calibration cast), None for others."""
+    if "bfloat16_copy_kernel" in name:
+        return "cast_f32_to_bf16"
+    if "la_sweep_pipe_kernel" in name:
+        m = re.search(r"Li(\d+)ELi(\d)ELb(\d)E", name) or re.search(r"<[^,]+, *(\d+), *(\d), *(true|false|0|1)", name)
+        if not m:
+            return "sweep_pipe"
+        rev = m.group(3) in ("1", "true")
+        wide = m.group(2) == "2"
+        return ("reverse" if rev else "forward") + ("_pair" if rev and wide else "_wide" if wide else "")
+    if "la_sweep_kernel" in name or "la_sweep_both_kernel" in name:
+        return "sweep_classic"
+    if "srms_fwd" in name:
+        return "srms_fwd"
+    if "srms_bwd" in name:
+        return "srms_bwd"
+    return None
+
+
+def counter_means(folder, counter):
+    vals = collections.defaultdict(list)
+    for path in glob.glob(os.path.join(folder, "**", "*counter_collection.csv"), recursive=True):
+        for r in csv.DictReader(open(path)):
+            key = classify(r["Kernel_Name"])
+            if key and r["Counter_Name"] == counter:
+                vals[key].append(float(r["Counter_Value"]))
+    # the cast runs on tensors of several sizes: keep the largest ones (the calibration size)
+    if vals.get("cast_f32_to_bf16"):
+        top = max(vals["cast_f32_to_bf16"])
+        vals["cast_f32_to_bf16"] = [v for v in vals["cast_f32_to_bf16"] if v > 0.9 * top]
+    return {k: statistics.fmean(v) for k, v in vals.items()}, {k: len(v) for k, v in vals.items()}
+
+
+def durations(folder):
+    vals = collections.defaultdict(list)
+    for path in glob.glob(os.path.join(folder, "**", "*kernel_trace.csv"), recursive=True):
+        for r in csv.DictReader(open(path)):
+            key = classify(r["Kernel_Name"])
+            if key:
+                vals[key].append((int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3)
+    return {k: {"calls": len(v), "avg_us": round(statistics.fmean(v), 1), "min_us": round(min(v), 1),
+                "median_us": round(statistics.median(v), 1), "max_us": round(max(v), 1)} for k, v in vals.items()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--kt")
+    ap.add_argument("--fetch")
+    ap.add_argument("--write")
+    ap.add_argument("--out", required=True)
+    a = ap.parse_args()
+    res = collections.defaultdict(dict)
+    if a.kt:
+        for k, v in durations(a.kt).items():
+            res[k]["duration"] = v
+    if a.fetch and a.write:
+        fetch, nf = counter_means(a.fetch, "FETCH_SIZE")
+        write, _ = counter_means(a.write, "WRITE_SIZE")
+        fs = CAST_READ / (fetch["cast_f32_to_bf16"] * 1024.0)
+        ws = CAST_WRITE / (write["cast_f32_to_bf16"] * 1024.0)
+        res["calibration"] = {"kernel": "float32 -> bfloat16 cast of [4,32,8192,128]", "fetch_scale": round(fs, 4),
+                              "write_scale": round(ws, 4), "FETCH_SIZE_KiB": round(fetch["cast_f32_to_bf16"], 1),
+                              "WRITE_SIZE_KiB": round(write["cast_f32_to_bf16"], 1)}
+        for k in fetch:
+            if k == "cast_f32_to_bf16" or k not in write:
+                continue
+            rd, wr = fetch[k] * 1024.0 * fs, write[k] * 1024.0 * ws
+            res[k].update({"FETCH_SIZE_KiB": round(fetch[k], 1), "WRITE_SIZE_KiB": round(write[k], 1),
+                           "read_bytes": round(rd), "write_bytes": round(wr), "hbm_bytes": round(rd + wr), "dispatches": nf[k]})
+    with open(a.out, "w") as f:
+        json.dump(res, f, indent=1, sort_keys=True)
+        f.write("\n")
+    print(json.dumps(res, indent=1, sort_keys=True))
+
+
+if __name__ == "__main__":
+    main()

@@ -5,13 +5,16 @@ parameter names (``q_proj, k_proj, v_proj, o_proj, norm, output_gate``) and arit
 state dict moves over unchanged.  What differs is data movement: the projections' ``(b, n, h*d)``
 outputs are handed to the operator as strided ``(b, h, n, d)`` views and its output comes back
 token-major, so neither the head split before the operator nor the head merge after it copies
-anything (the reference's two ``rearrange`` calls, :56-64, each end in a copy kernel).
+anything (the reference's two ``rearrange`` calls, :56-64, each end in a copy kernel), and the
+output LayerNorm, the sigmoid of the gate and their product (:66-69) are one fused row kernel
+(``lightning_attn.ops.hip.norm_gate``) where the embedding width allows it.
 """
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
 from lightning_attn.ops import lightning_attn_func
+from lightning_attn.ops.hip import norm_gate, norm_gate_supported
 from lightning_attn.utils import _build_slope_tensor
 
 
@@ -33,6 +36,7 @@ class TnlAttention(nn.Module):
         # per-head decay rates, shrinking towards the last layer (tnl_attn.py:36-38)
         depth_scale = 1 - layer_idx / (num_layers - 1) + 1e-5
         self.register_buffer("slope_rate", _build_slope_tensor(num_heads) * depth_scale, persistent=False)
+        self.fused_norm_gate = True  # False: LayerNorm, sigmoid and product as separate PyTorch operators
 
     def _heads(self, t):
         """(b, n, h*d) -> (b, h, n, d) as a view."""
@@ -42,8 +46,10 @@ class TnlAttention(nn.Module):
         q, k, v = (self._heads(F.silu(proj(x))) for proj in (self.q_proj, self.k_proj, self.v_proj))
         mixed = lightning_attn_func(q, k, v, self.slope_rate)  # (b, h, n, d), token-major memory
         mixed = mixed.transpose(-3, -2).flatten(-2)            # (b, n, h*d): a view of that memory
-        gate = torch.sigmoid(self.output_gate(x))
-        return self.o_proj(self.norm(mixed) * gate)
+        gate = self.output_gate(x)
+        if self.fused_norm_gate and mixed.is_cuda and norm_gate_supported(mixed.shape[-1], mixed.dtype):
+            return self.o_proj(norm_gate(mixed, gate, self.norm.weight, self.norm.bias, self.norm.eps))
+        return self.o_proj(self.norm(mixed) * torch.sigmoid(gate))
 
 
 if __name__ == "__main__":

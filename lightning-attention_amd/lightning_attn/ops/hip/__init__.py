@@ -7,3 +7,4 @@ from .lightning_attn2 import (  # noqa: F401
 )
 from .srmsnorm import SimpleRMSNorm, _SrmsNorm  # noqa: F401
 from ._lib import launch_opts  # noqa: F401
+from .norm_gate import norm_gate, norm_gate_supported  # noqa: F401

@@ -19,7 +19,7 @@ SYMBOLS = (
     "la_version", "la_error_string", "la_supported", "la_workspace_bytes",
     "la_fwd", "la_bwd", "la_fwd_strided", "la_bwd_strided", "la_workspace_bytes_opts", "la_fwd_opts", "la_bwd_opts",
     "la_fwd_static",
-    "srmsnorm_fwd", "srmsnorm_bwd",
+    "srmsnorm_fwd", "srmsnorm_bwd", "norm_gate_supported", "norm_gate_workspace_bytes", "norm_gate_fwd", "norm_gate_bwd",
 )
 
 _lib = None
@@ -109,6 +109,14 @@ def lib():
             L.srmsnorm_fwd.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _f, _int, _vp]
             L.srmsnorm_bwd.restype = _int
             L.srmsnorm_bwd.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]
+            L.norm_gate_supported.restype = _int
+            L.norm_gate_supported.argtypes = [_i64, _int]
+            L.norm_gate_workspace_bytes.restype = _sz
+            L.norm_gate_workspace_bytes.argtypes = [_i64, _i64, _int]
+            L.norm_gate_fwd.restype = _int
+            L.norm_gate_fwd.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f, _int, _vp]
+            L.norm_gate_bwd.restype = _int
+            L.norm_gate_bwd.argtypes = [_vp] * 11 + [_vp, _sz, _i64, _i64, _int, _vp]
             _lib = L
     return _lib
 

@@ -1,0 +1,69 @@
+"""Gated output norm of the TNL attention block over the HIP row kernels:
+``norm_gate(o, g, weight, bias, eps) = layer_norm(o, weight, bias, eps) * sigmoid(g)``,
+the arithmetic of the reference's examples/module/tnl_attn.py:66-69 in one pass forward and
+one backward."""
+import torch
+
+from . import _lib
+
+
+def norm_gate_supported(cols, dtype):
+    """True when the kernels take rows of `cols` elements of `dtype`."""
+    try:
+        code = _lib.dtype_code(dtype)
+    except TypeError:
+        return False
+    return bool(_lib.lib().norm_gate_supported(cols, code))
+
+
+class _NormGate(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, o, g, weight, bias, eps):
+        _lib.require_same_device("norm_gate", o=o, g=g, weight=weight, bias=bias)
+        if not (o.dtype == g.dtype == weight.dtype == bias.dtype):
+            raise TypeError("o, g, weight and bias must share a dtype")
+        cols = o.shape[-1]
+        if g.shape != o.shape or weight.shape != (cols,) or bias.shape != (cols,):
+            raise ValueError("shape mismatch: o %s g %s weight %s bias %s"
+                             % (tuple(o.shape), tuple(g.shape), tuple(weight.shape), tuple(bias.shape)))
+        code = _lib.dtype_code(o.dtype)
+        o2, g2 = o.reshape(-1, cols).contiguous(), g.reshape(-1, cols).contiguous()
+        weight, bias = weight.contiguous(), bias.contiguous()
+        rows = o2.shape[0]
+        y = torch.empty_like(o2)
+        mean = torch.empty((rows,), dtype=torch.float32, device=o.device)
+        rstd = torch.empty((rows,), dtype=torch.float32, device=o.device)
+        with _lib.on_device(o.device):
+            rc = _lib.lib().norm_gate_fwd(o2.data_ptr(), g2.data_ptr(), weight.data_ptr(), bias.data_ptr(), y.data_ptr(),
+                                          mean.data_ptr(), rstd.data_ptr(), rows, cols, float(eps), code,
+                                          _lib.stream_ptr(o.device))
+        _lib.check(rc, "norm_gate_fwd")
+        ctx.save_for_backward(o2, g2, weight, bias, mean, rstd)
+        ctx.shape = o.shape
+        return y.reshape(o.shape)
+
+    @staticmethod
+    def backward(ctx, dy):
+        o2, g2, weight, bias, mean, rstd = ctx.saved_tensors
+        rows, cols = o2.shape
+        if dy.device != o2.device:
+            raise RuntimeError("norm_gate backward: the upstream gradient is on %s, the inputs on %s" % (dy.device, o2.device))
+        dy2 = dy.to(o2.dtype).reshape(rows, cols).contiguous()
+        code = _lib.dtype_code(o2.dtype)
+        d_o, d_g = torch.empty_like(o2), torch.empty_like(g2)
+        dw, db = torch.empty_like(weight), torch.empty_like(bias)
+        L = _lib.lib()
+        with _lib.on_device(o2.device):
+            ws_bytes = L.norm_gate_workspace_bytes(rows, cols, code)
+            ws = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=o2.device)
+            rc = L.norm_gate_bwd(o2.data_ptr(), g2.data_ptr(), weight.data_ptr(), bias.data_ptr(), mean.data_ptr(),
+                                 rstd.data_ptr(), dy2.data_ptr(), d_o.data_ptr(), d_g.data_ptr(), dw.data_ptr(), db.data_ptr(),
+                                 ws.data_ptr(), ws_bytes, rows, cols, code, _lib.stream_ptr(o2.device))
+        _lib.check(rc, "norm_gate_bwd")
+        return d_o.reshape(ctx.shape), d_g.reshape(ctx.shape), dw, db, None
+
+
+def norm_gate(o, g, weight, bias, eps=1e-5):
+    """layer_norm(o, (C,), weight, bias, eps) * sigmoid(g) over the last dim; differentiable in
+    o, g, weight and bias.  HIP tensors only; see norm_gate_supported for the row widths."""
+    return _NormGate.apply(o, g, weight, bias, eps)

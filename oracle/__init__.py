@@ -24,3 +24,4 @@ from .linear_attn_oracle import (  # noqa: F401
     block_recurrence_bwd,
 )
 from .srmsnorm_oracle import srmsnorm, srmsnorm_fwd_bwd, srmsnorm_f64  # noqa: F401
+from .norm_gate_oracle import norm_gate as norm_gate_ref, norm_gate_fwd_bwd, norm_gate_closed_form  # noqa: F401

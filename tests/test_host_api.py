@@ -17,7 +17,7 @@ HEADER = os.path.join(ROOT, "include", "lightning_attn_hip.h")
 def _declared_symbols():
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b((?:la|srmsnorm)_[a-z_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b((?:la|srmsnorm|norm_gate)_[a-z_]+)\s*\(", text)))
 
 
 def test_library_exports_every_declared_symbol():
