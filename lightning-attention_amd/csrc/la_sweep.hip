@@ -86,7 +86,7 @@ __device__ __forceinline__ void sweep_body(const SweepPair& pair, const unsigned
     const __amdgpu_buffer_rsrc_t ob = seq_rsrc<T>(a.out, a.lo, unit, a.h, n, dv);
     const unsigned xts = (unsigned)a.lx.ts, yts = (unsigned)a.ly.ts, zts = (unsigned)a.lz.ts, ots = (unsigned)a.lo.ts;
     const unsigned nrows = (unsigned)n;
-    const int col0 = slice * 64;
+    const int col0 = slice * 64;  // (a.zw is 64 for this kernel)
     const bool cols_active = (col0 + 16 * w) < dv;
 
     float rate = 0.f;
@@ -578,6 +578,7 @@ static SweepArgs make_args(const SweepIO& io, const float* s, int64_t bh, int64_
     a.lx = io.lx; a.ly = io.ly; a.lz = io.lz; a.lo = io.lo;
     a.n = n; a.dk = (int)dk; a.dv = (int)dv; a.h = (int)h; a.bh = (int)bh;
     a.nslice = (int)((dv + 63) / 64);
+    a.zw = 64;
     return a;
 }
 
@@ -619,13 +620,24 @@ struct ScanPlan {
 // into the state.  Warm-up blocks: with the geometric chunk lengths of choose_chunks the longest
 // workgroup runs the fraction `frac` of a single walk.  Scanned states: a chunk one and a half times,
 // plus two more launches and the scan (16 us measured, and 10 for the host's share).
-static double block_us(int64_t dk, bool wide) { return dk <= 64 ? 1.0 : dk <= 128 ? (wide ? 1.75 : 1.4) : dk <= 192 ? 2.1 : 2.9; }
+static double block_us(int64_t dk, bool wide) {
+    if (dk <= 64) return 1.0;
+    if (dk <= 128) return wide ? 1.75 : 1.4;
+    if (dk <= 192) return wide ? 3.0 : 2.1;
+    return wide ? 4.1 : 2.9;
+}
+// Column slices per sequence: 64 columns each, or - wide - 128 (feature dim up to 128), 96 (up to 192), 128 (up to 256).
+static int64_t wide_slices(int64_t dk, int64_t dv) {
+    const int64_t zw = dk <= 128 ? 128 : wide_zw_max((int)dk);
+    return (dv + zw - 1) / zw;
+}
+static int64_t slices(int64_t dk, int64_t dv, bool wide) { return wide ? wide_slices(dk, dv) : (dv + 63) / 64; }
 static double warm_up_frac(int64_t wgs, int64_t nblk) {
     static const double frac[9] = {1.0, 1.0, 0.77, 0.71, 0.68, 0.67, 0.66, 0.66, 0.66};
     return frac[warm_up_chunks(wgs, nblk)];
 }
 static double warm_up_us(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, bool wide) {
-    const int64_t nblk = (n + 63) / 64, wgs = (bh + 7) / 8 * 8 * (wide ? 1 : (dv + 63) / 64) * nprod;
+    const int64_t nblk = (n + 63) / 64, wgs = (bh + 7) / 8 * 8 * slices(dk, dv, wide) * nprod;
     return warm_up_frac(wgs, nblk) * (double)nblk * block_us(dk, wide);
 }
 
@@ -635,7 +647,7 @@ static ScanPlan plan_scan(int64_t bh, int64_t n, int64_t dk, int64_t dv, int npr
     if (opts.scan == LA_OPT_OFF) return none;
     const int forced = opts.chunks;
     const int64_t nblk = (n + 63) / 64, cus = num_cus();
-    const int64_t nslice = wide ? 1 : (dv + 63) / 64;
+    const int64_t nslice = slices(dk, dv, wide);
     const int64_t wgs = (bh + 7) / 8 * 8 * nslice * nprod;
     int64_t c = 1;
     if (forced > 0) c = forced;
@@ -662,7 +674,19 @@ static ScanPlan plan_scan(int64_t bh, int64_t n, int64_t dk, int64_t dv, int npr
 // 64-column one, and there are half as many: compare the rounds of workgroups the chip has to run.
 // `scratch`: bytes of workspace the caller has.  opts.wide overrides the choice.
 static bool wide_columns(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, size_t scratch, const Opts& opts) {
-    if (dk > 128 || dv <= 64 || dv > 128) return false;
+    if (dk > 128) {
+        // Two-barrier kernels: 96- / 128-column workgroups (la_sweep_wide.hip) where that makes fewer slices.
+        // They pay when the 64-column form needs more rounds of workgroups than the chip has CUs for
+        // (a wide workgroup takes about 1.4 times as long); with few sequences the 64-column form has
+        // more workgroups to spread over the CUs and stays.
+        const int64_t ws = wide_slices(dk, dv), ns = (dv + 63) / 64;
+        if (ws >= ns) return false;
+        if (opts.wide != LA_OPT_AUTO) return opts.wide == LA_OPT_ON;
+        const int64_t cus = num_cus(), units = (bh + 7) / 8 * 8 * nprod, wide = units * ws, narrow = units * ns;
+        if (narrow <= cus) return false;
+        return (wide + cus - 1) / cus * 7 < (narrow + cus - 1) / cus * 5;
+    }
+    if (dv <= 64 || dv > 128) return false;
     if (opts.wide != LA_OPT_AUTO) return opts.wide == LA_OPT_ON;
     if (dk <= 64) return false;  // the 128-column form pads the feature dim to 128
     const int64_t cus = num_cus(), wide = (bh + 7) / 8 * 8 * nprod, narrow = 2 * wide;
@@ -691,7 +715,12 @@ static int launch_planned(SweepPair& p, int64_t bh, int64_t n, int64_t dk, int64
     p.chunk_len = 0;
     p.state = nullptr;
     for (int i = 0; i < p.nprod; ++i)
-        if (p.wide) p.a[i].nslice = 1;
+        if (p.wide) {
+            const int64_t ws = wide_slices(dk, dv);
+            p.a[i].nslice = (int)ws;
+            // equal slices, a whole number of 32-column state waves each
+            p.a[i].zw = dk <= 128 ? 128 : (int)(((dv + ws - 1) / ws + 31) / 32 * 32);
+        }
     const ScanPlan pl = plan_scan(bh, n, dk, dv, p.nprod, p.wide != 0, opts);
     if (pl.nchunk > 1 && ws_ok && ws_bytes >= pl.bytes) {
         p.mode = kCollect;  // sweep_pipe runs the three launches
@@ -710,6 +739,7 @@ static int launch_planned(SweepPair& p, int64_t bh, int64_t n, int64_t dk, int64
     }
     if (p.nprod == 1) p.a[1] = p.a[0];
     if (dk <= 128) return sweep_pipe(p, dtype, reverse, st);  // pipelined kernel, la_sweep_pipe.hip
+    if (p.wide) return sweep_wide(p, dtype, reverse, st);     // 96- / 128-column workgroups, la_sweep_wide.hip
     return launch_classic(p, dtype, reverse, st);
 }
 

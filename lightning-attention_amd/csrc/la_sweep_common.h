@@ -24,6 +24,7 @@ struct SweepArgs {
     const float* s; // h decay rates or nullptr
     int64_t n;
     int dk, dv, h, bh, nslice;
+    int zw;              // columns of z / out per slice (la_sweep.hip: 64; la_sweep_wide.hip: a multiple of 32 up to 128)
     int nchunk;          // sequence chunks per (batch, head, slice); 1 = one workgroup walks the whole sequence
     int chunk_start[9];  // first 64-token block (in walk order) of each chunk; chunk_start[nchunk] = number of blocks
 };
@@ -161,5 +162,9 @@ inline size_t pipe_state_floats(int dk, bool wide) {
 }
 // Between a kCollect and a kApply launch: scans the chunks' end states in place (la_sweep_pipe.hip).
 int launch_state_scan(const SweepPair& p, hipStream_t st);
+// Launches the two-barrier kernel with 96- / 128-column workgroups (feature dims 129 .. 256); la_sweep_wide.hip.
+int sweep_wide(const SweepPair& p, int dtype, bool reverse, hipStream_t st);
+// Columns per workgroup that kernel can take at a feature dim.
+inline int wide_zw_max(int dk) { return dk <= 192 ? 96 : 128; }
 
 }  // namespace la

@@ -2,7 +2,8 @@
 
 The reference pads e to a power of two and splits d > 128 into <= 64-wide
 slices because its Triton tiles need that; the HIP kernels tile any multiple of
-8 up to 256 natively (128 for float32), so neither happens here.  Larger feature
+8 up to 256 natively (128 for float32), so neither happens here (other sizes are
+zero-padded to the next multiple of 8, which is exact).  Larger feature
 dims are split into slices of q/k whose partial outputs add up (the scores are
 additive over feature slices) and into column groups of v."""
 import torch
@@ -13,8 +14,17 @@ _VARIANTS = ("chunk_loop", "parallel")
 
 
 def is_support(dim):
-    """True when a feature dim is usable: a positive multiple of 8."""
-    return dim > 0 and dim % 8 == 0
+    """True when a feature dim is usable: any positive size.  Multiples of 8 run as they are, other
+    sizes are zero-padded to the next multiple of 8 (the reference's gate, ``16 % dim``, rejects the
+    divisors of 16 and pads e to a power of two, lightning_attn_interface.py:8-9, 29-33)."""
+    return dim > 0
+
+
+def _pad8(t):
+    """Last dim zero-padded to the next multiple of 8: zero features add nothing to q . k, zero
+    columns of v give zero columns of o."""
+    extra = -t.shape[-1] % 8
+    return torch.nn.functional.pad(t, (0, extra)) if extra else t
 
 
 def lightning_attn_func(q, k, v, s=None, variant="chunk_loop"):
@@ -27,7 +37,9 @@ def lightning_attn_func(q, k, v, s=None, variant="chunk_loop"):
         raise ValueError("variant must be one of %s, got %r" % (_VARIANTS, variant))
     b, h, n, d = q.shape
     e = v.shape[-1]
-    assert is_support(d) and is_support(e), "feature dims must be multiples of 8 (got d=%d, e=%d)" % (d, e)
+    assert is_support(d) and is_support(e), "feature dims must be positive (got d=%d, e=%d)" % (d, e)
+    if d % 8 or e % 8:
+        return lightning_attn_func(_pad8(q), _pad8(k), _pad8(v), s, variant)[..., :e]
 
     _MAX_DIM = 128 if q.dtype == torch.float32 else 256
 

@@ -552,3 +552,53 @@ def test_tensors_on_different_devices_are_refused():
         lightning_attn_func(q.to(DEV), k, v.to(DEV), None)
     with pytest.raises(RuntimeError, match="same HIP device"):
         lightning_attn2(q.to(DEV), k.to(DEV), v, _build_slope_tensor(2).to(DEV))
+
+
+@pytest.mark.parametrize("b, h, n, d, e, dtype", [(1, 3, 300, 64, 100, torch.bfloat16), (2, 2, 130, 36, 36, torch.bfloat16),
+                                                  (1, 2, 257, 20, 12, torch.float32), (1, 1, 70, 100, 260, torch.float16)])
+def test_feature_dims_off_the_grid_of_8_are_padded(b, h, n, d, e, dtype):
+    """d or e not a multiple of 8 (the reference takes any e by padding v to a power of two,
+    lightning_attn_interface.py:29-33, 63-64): zero-padded to the next multiple of 8, gradients sliced back."""
+    q, k, v, do = make_inputs(b, h, n, d, e, dtype, 0.5, seed=d * e)
+    s = _build_slope_tensor(h)
+    want = oracle.linear_attn_fwd_bwd(q, k, v, s, do, torch.float64 if dtype == torch.float32 else torch.float32)
+    got = run_hip(q, k, v, s, do)
+    for a, t in zip(got, (v, q, k, v)):
+        assert a.shape == t.shape
+    check(got, want, dtype, "padded dims %s" % ((b, h, n, d, e),))
+
+
+@pytest.mark.parametrize("b, h, n, d, e", [(2, 3, 700, 192, 192), (1, 2, 450, 256, 256), (1, 3, 513, 160, 160), (2, 2, 300, 136, 200),
+                                           (1, 2, 330, 192, 256), (1, 1, 200, 256, 72), (1, 2, 260, 144, 96), (1, 2, 1000, 224, 232)])
+@pytest.mark.parametrize("decay", [True, False])
+def test_wide_two_barrier_kernel_is_bit_identical_to_the_64_column_form(b, h, n, d, e, decay):
+    """Feature dims above 128: 96- / 128-column workgroups (wide=True) against the 64-column ones (wide=False), forward
+    and backward, single walk, warm-up chunks and - d == e - the paired dK + dV launch: the same arithmetic per output
+    column, so the same bits; from scanned chunk states equal to rounding.  Both against the oracle."""
+    q, k, v, do = make_inputs(b, h, n, d, e, torch.bfloat16, 0.7, seed=d + e)
+    s = _build_slope_tensor(h) if decay else None
+    narrow = run_hip(q, k, v, s, do, wide=False, scan=False, chunks=1, once=False)
+    want = oracle.linear_attn_fwd_bwd(q, k, v, s, do, torch.float32)
+    check(narrow, want, torch.bfloat16, "64-column %s" % ((b, h, n, d, e),))
+    for opts in ({"chunks": 1}, {"chunks": 3}, {"chunks": 2, "paired": False}):
+        wide = run_hip(q, k, v, s, do, wide=True, scan=False, once=False, **opts)
+        for name, a, c in zip(("o", "dq", "dk", "dv"), wide, narrow):
+            assert torch.equal(a, c), (opts, name)
+    scanned = run_hip(q, k, v, s, do, wide=True, chunks=4, once=False)
+    for name, a, c in zip(("o", "dq", "dk", "dv"), scanned, narrow):
+        assert rel_norm(a, c) < 5e-4, name
+    check(scanned, want, torch.bfloat16, "wide, scanned chunks %s" % ((b, h, n, d, e),))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_many_sequences_at_192_take_the_wide_workgroups(dtype):
+    """b * h = 48 sequences at d = e = 192: three 64-column workgroups per sequence would not fit the CUs in one
+    round (a chip of 256 of them is assumed when there are fewer), so the library picks two 96-column ones by itself."""
+    b, h, n, d = 6, 16, 200, 192
+    q, k, v, do = make_inputs(b, h, n, d, d, dtype, 0.5, seed=5)
+    s = _build_slope_tensor(h)
+    want = oracle.linear_attn_fwd_bwd(q, k, v, s, do, torch.float32)
+    got = run_hip(q, k, v, s, do)
+    check(got, want, dtype, "many sequences, d = 192")
+    for a, c in zip(got, run_hip(q, k, v, s, do, wide=False)):
+        assert torch.equal(a, c)

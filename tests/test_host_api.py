@@ -198,9 +198,9 @@ def test_no_cpu_fallback():
 
 
 def test_interface_validation():
-    q = torch.randn(1, 2, 16, 12)
+    q = torch.randn(1, 2, 16, 0)
     with pytest.raises(AssertionError):
-        lightning_attn_func(q, q, q)  # d = 12 is not a multiple of 8
+        lightning_attn_func(q, q, q)  # no features at all
     with pytest.raises(ValueError):
         lightning_attn_func(torch.randn(1, 2, 16, 16), torch.randn(1, 2, 16, 16), torch.randn(1, 2, 16, 16), None, "ring")
 
@@ -210,3 +210,20 @@ def test_missing_library_is_an_error(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/liblightning_attn_hip.so")
     with pytest.raises(RuntimeError, match="not built"):
         _lib.lib()
+
+
+def test_triton_import_path_is_an_alias_of_the_hip_operators():
+    """lightning_attn/ops/triton/__init__.py:1-4 of the reference exports its operators under
+    lightning_attn.ops.triton; the same imports work here and name the HIP operators."""
+    from lightning_attn.ops import hip
+    from lightning_attn.ops.triton import SimpleRMSNorm as S1, lightning_attn2 as a1, lightning_attn2_no_decay as a2
+    from lightning_attn.ops.triton import lightning_attn2_parallel as a3
+    from lightning_attn.ops.triton.lightning_attn2 import LightningAttention2, lightning_attn2 as b1
+    from lightning_attn.ops.triton.lightning_attn2_no_decay import lightning_attn2_no_decay as b2
+    from lightning_attn.ops.triton.lightning_attn2_parallel import lightning_attn2_parallel as b3
+    from lightning_attn.ops.triton.srmsnorm import SimpleRMSNorm as S2, _SrmsNorm
+    assert S1 is hip.SimpleRMSNorm and S2 is S1 and _SrmsNorm is hip._SrmsNorm
+    assert LightningAttention2 is hip.LightningAttention2
+    for f in (a1, a2, a3, b1, b2, b3):
+        assert callable(f)
+    assert a1.__self__ is hip.LightningAttention2 and a2.__self__ is hip.LightningAttention2NoDecay
