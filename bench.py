@@ -212,6 +212,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--no-sweep", action="store_true", help="skip the fwd/bwd split, the n sweep and the other configurations")
     ap.add_argument("--no-srms", action="store_true", help="skip the SRMSNorm timings")
+    ap.add_argument("--shape", default=None, metavar="B,H,N,D",
+                    help="not the benchmark: run only W + K forward+backward steps at this shape (bf16, d = e) and print "
+                         "their event timings; for profiling the kernels of other shapes under rocprofv3")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU part (every (batch, head) sequence is "
@@ -232,6 +235,21 @@ def main():
     def inputs(n):
         q, k, v, do = (torch.randn(B, H, n, D, device=dev, dtype=torch.float32).bfloat16() for _ in range(4))
         return q.requires_grad_(), k.requires_grad_(), v.requires_grad_(), do
+
+    if args.shape:
+        b_, h_, n_, d_ = (int(t) for t in args.shape.split(","))
+        s_ = _build_slope_tensor(h_).to(dev).to(torch.float32)
+        q, k, v, do = (torch.randn(b_, h_, n_, d_, device=dev, dtype=torch.float32).bfloat16() for _ in range(4))
+        q, k, v = q.requires_grad_(), k.requires_grad_(), v.requires_grad_()
+
+        def shape_step():
+            lightning_attn_func(q, k, v, s_).backward(do)
+            q.grad = k.grad = v.grad = None
+
+        ms, ev_ts = timed_steps(shape_step, args.warmup, args.steps)
+        print(json.dumps({"metric": "profiling run, not the benchmark", "shape": [b_, h_, n_, d_], "dtype": "bf16",
+                          "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "step_event_ms": stats(ev_ts)}))
+        return
 
     s = _build_slope_tensor(H).to(dev).to(torch.float32)
     q, k, v, do = inputs(N)

@@ -3,7 +3,7 @@ with the output norm, sigmoid gate and product fused into one row kernel (``norm
 separate PyTorch operators of the reference's block (tnl_attn.py:66-69), and the time of the fused kernel
 against that chain on its own.
 
-    python lightning-attention_amd/benchmarks/benchmark_tnl_block.py [--quick]
+    python lightning-attention_amd/benchmarks/benchmark_tnl_block.py [--quick | --large]
 
 Under ``rocprofv3 --kernel-trace --stats`` the same run gives the split of the block by kernel (projection
 GEMMs, the three SiLU passes, the attention sweeps, the norm / gate kernels).
@@ -32,6 +32,8 @@ def main():
     dev = torch.device("cuda")
     torch.manual_seed(2024)
     shapes = [(2, 2048, 1024, 8)] if quick else [(2, 2048, 1024, 8), (4, 4096, 2048, 16), (4, 8192, 4096, 32)]
+    if "--large" in sys.argv:  # the block around the benchmark shape of the operator only
+        shapes = shapes[-1:]
     print("TNL block, bf16: b, n, embed, heads | block fwd+bwd ms, fused norm-gate / separate operators | "
           "norm-gate alone fwd, bwd ms: fused / separate")
     for b, n, embed, heads in shapes:

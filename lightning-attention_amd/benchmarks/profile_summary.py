@@ -10,8 +10,9 @@ traffic per launch from the FETCH_SIZE / WRITE_SIZE counters.
         --out REPO/profiles/la_step_b4_h32_n8192_d128_bf16.counters.json
 
 Both counters report KiB per dispatch.  They are scaled by what they read for a kernel of known
-size in the same run: PyTorch's float32 -> bfloat16 cast of a [4, 32, 8192, 128] tensor (bench.py
-makes its inputs that way), which reads 512 MiB and writes 256 MiB.
+size in the same run: PyTorch's float32 -> bfloat16 cast of the run's largest tensor (bench.py
+makes its inputs that way; [4, 32, 8192, 128] unless --cast-elements says otherwise), which reads
+4 and writes 2 bytes per element.  The run must not hold larger casts (so: --no-sweep, or --shape).
 """
 import argparse
 import collections
@@ -22,8 +23,7 @@ import os
 import re
 import statistics
 
-CAST_READ = 4 * 32 * 8192 * 128 * 4
-CAST_WRITE = 4 * 32 * 8192 * 128 * 2
+CAST_ELEMENTS = 4 * 32 * 8192 * 128  # the largest tensor bench.py casts in a --no-sweep run
 
 
 def classify(name):
@@ -37,8 +37,23 @@ def classify(name):
         rev = m.group(3) in ("1", "true")
         wide = m.group(2) == "2"
         return ("reverse" if rev else "forward") + ("_pair" if rev and wide else "_wide" if wide else "")
-    if "la_sweep_kernel" in name or "la_sweep_both_kernel" in name:
+    if "la_sweep_wide_kernel" in name:
+        m = re.search(r"Li(\d+)ELb(\d)E", name) or re.search(r"<[^,]+, *(\d+), *(true|false|0|1)", name)
+        return "sweep_wide%s_%s" % (m.group(1), "reverse" if m.group(2) in ("1", "true") else "forward") if m else "sweep_wide"
+    if "la_sweep_both_kernel" in name or "la_sweep_pipe_both_kernel" in name:
+        return "sweep_both"
+    if "la_sweep_kernel" in name:
         return "sweep_classic"
+    if "la_state_scan" in name:
+        return "state_scan"
+    if "norm_gate_fwd" in name:
+        return "norm_gate_fwd"
+    if "norm_gate_bwd" in name:
+        return "norm_gate_bwd"
+    if "norm_gate_reduce" in name:
+        return "norm_gate_reduce"
+    if "silu" in name.lower():
+        return "torch_silu_bwd" if "backward" in name.lower() else "torch_silu"
     if "srms_fwd" in name:
         return "srms_fwd"
     if "srms_bwd" in name:
@@ -77,7 +92,9 @@ def main():
     ap.add_argument("--fetch")
     ap.add_argument("--write")
     ap.add_argument("--out", required=True)
+    ap.add_argument("--cast-elements", type=int, default=CAST_ELEMENTS)
     a = ap.parse_args()
+    cast_read, cast_write = 4 * a.cast_elements, 2 * a.cast_elements
     res = collections.defaultdict(dict)
     if a.kt:
         for k, v in durations(a.kt).items():
@@ -85,9 +102,9 @@ def main():
     if a.fetch and a.write:
         fetch, nf = counter_means(a.fetch, "FETCH_SIZE")
         write, _ = counter_means(a.write, "WRITE_SIZE")
-        fs = CAST_READ / (fetch["cast_f32_to_bf16"] * 1024.0)
-        ws = CAST_WRITE / (write["cast_f32_to_bf16"] * 1024.0)
-        res["calibration"] = {"kernel": "float32 -> bfloat16 cast of [4,32,8192,128]", "fetch_scale": round(fs, 4),
+        fs = cast_read / (fetch["cast_f32_to_bf16"] * 1024.0)
+        ws = cast_write / (write["cast_f32_to_bf16"] * 1024.0)
+        res["calibration"] = {"kernel": "float32 -> bfloat16 cast of %d elements" % a.cast_elements, "fetch_scale": round(fs, 4),
                               "write_scale": round(ws, 4), "FETCH_SIZE_KiB": round(fetch["cast_f32_to_bf16"], 1),
                               "WRITE_SIZE_KiB": round(write["cast_f32_to_bf16"], 1)}
         for k in fetch:
