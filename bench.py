@@ -74,9 +74,41 @@ def event_times(fn, reps, warm=3):
     return [ev[i].elapsed_time(ev[i + 1]) for i in range(reps)]
 
 
-def event_ms(fn, reps, warm=3):
-    """Median per-call duration (ms)."""
-    return statistics.median(event_times(fn, reps, warm))
+def event_times_timed(fn, warm_ms=60.0, rep_ms=100.0, batch_ms=2.0):
+    """Per-call durations (ms) with warm-up and repetitions by time, as in the reference's protocol
+    (triton.testing.do_bench in benchmarks/benchmark_lightning2.py:97-118), with two differences that matter on
+    this chip: the warm-up is 60 ms (after a change of shape the clocks need 20-30 ms under load to settle), and
+    calls shorter than `batch_ms` are timed in batches between one pair of events, so that no event record sits
+    between two short launches."""
+    import torch
+
+    fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(3):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    est = max(e0.elapsed_time(e1) / 3, 1e-3)
+    for _ in range(max(5, int(warm_ms / est))):
+        fn()
+    per = max(1, int(batch_ms / est))            # calls per batch
+    nb = max(10, int(rep_ms / (est * per)))      # batches
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(nb + 1)]
+    torch.cuda.synchronize()
+    ev[0].record()
+    for i in range(nb):
+        for _ in range(per):
+            fn()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    return [ev[i].elapsed_time(ev[i + 1]) / per for i in range(nb)]
+
+
+def event_ms(fn, reps=None, warm=None):
+    """Median per-call duration (ms), warm-up and repetitions by time."""
+    return statistics.median(event_times_timed(fn))
 
 
 def stats(ts):
@@ -331,14 +363,14 @@ def main():
             o.backward(do, retain_graph=True)
             q.grad = k.grad = v.grad = None
 
-        out["fwd_ms"] = stats(event_times(lambda: lightning_attn_func(q, k, v, s), 20))
-        out["bwd_ms"] = stats(event_times(bwd_only, 20))
+        out["fwd_ms"] = stats(event_times_timed(lambda: lightning_attn_func(q, k, v, s)))
+        out["bwd_ms"] = stats(event_times_timed(bwd_only))
         del o
         sweep, prev = {}, None
         for n in (512, 1024, 2048, 4096, 8192, 16384, 32768):
             q = k = v = do = None
             q, k, v, do = inputs(n)
-            ts = event_times(step, 10 if n >= 16384 else 20, warm=5)
+            ts = event_times_timed(step)
             med = statistics.median(ts)
             sweep[str(n)] = {"median": round(med, 4), "min": round(min(ts), 4),
                              "ratio_to_half_n": round(med / prev, 3) if prev else None}
@@ -395,8 +427,8 @@ def main():
             y.backward(dy, retain_graph=True)
             x.grad = None
 
-        f_ts = event_times(lambda: norm(x), 50)
-        b_ts = event_times(nbwd, 50)
+        f_ts = event_times_timed(lambda: norm(x))
+        b_ts = event_times_timed(nbwd)
         f_ms, b_ms = statistics.median(f_ts), statistics.median(b_ts)
         fbytes, bbytes = rows * (2 * 2 * cols + 4), rows * (3 * 2 * cols + 4)
         out["srmsnorm"] = {

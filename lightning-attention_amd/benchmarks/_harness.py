@@ -1,7 +1,9 @@
 """Timing / memory harness for the benchmark tables (no Triton): same protocol as the
-``triton.testing.do_bench`` calls in the reference's benchmarks (warm-up for >= 25 ms, then
+``triton.testing.do_bench`` calls in the reference's benchmarks (warm-up by time, then
 repetitions for >= 100 ms, gradients cleared between repetitions, median of per-call times
-taken with device events)."""
+taken with device events).  The warm-up is 60 ms instead of the reference's 25: coming out of idle,
+or after a change of shape, the chip's clocks take 20-30 ms under load to settle, and short calls
+measured inside that window read up to twice their steady time."""
 import statistics
 
 import torch
@@ -9,7 +11,7 @@ import torch
 from lightning_attn.utils import get_memory
 
 
-def do_bench(fn, warmup_ms=25.0, rep_ms=100.0, grads=()):
+def do_bench(fn, warmup_ms=60.0, rep_ms=100.0, grads=()):
     fn()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

@@ -280,6 +280,12 @@ __device__ __forceinline__ void sweep_wide_body(const SweepPair& pair, const uns
                         if (need) bp[i4][ks] = *reinterpret_cast<const V8*>(Ps + (16 * i4 + r) * PS + 32 * ks + 8 * g);
                     }
                 }
+                // the inter-block tiles of both slabs first: their place in LDS then takes this wave's output tile
+                f32x4 oacc[NH][4];
+#pragma unroll
+                for (int h = 0; h < NH; ++h)
+#pragma unroll
+                    for (int i4 = 0; i4 < 4; ++i4) oacc[h][i4] = Ob[((w * NH + h) * 4 + i4) * 64 + lane];
 #pragma unroll
                 for (int h = 0; h < NH; ++h) {
                     if (col0 + cbase + 16 * h >= colend) continue;
@@ -289,27 +295,43 @@ __device__ __forceinline__ void sweep_wide_body(const SweepPair& pair, const uns
                         const T* pz = Zs + (32 * ks + 8 * g + (r >> 2)) * ZS + cbase + 16 * h + 4 * (r & 3);
                         zf[ks] = cat<V8, V4>(lds_tr4<V4>(pz), lds_tr4<V4>(pz + 4 * ZS));
                     }
-                    f32x4 oacc[4];
-#pragma unroll
-                    for (int i4 = 0; i4 < 4; ++i4) oacc[i4] = Ob[((w * NH + h) * 4 + i4) * 64 + lane];
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int i4 = 0; i4 < 4; ++i4) {
 #pragma unroll
                         for (int ks = 0; ks < 2; ++ks) {
                             const bool need = REVERSE ? (ks >= i4 / 2) : (ks <= i4 / 2);
-                            if (need) oacc[i4] = M::mma(zf[ks], bp[i4][ks], oacc[i4]);
+                            if (need) oacc[h][i4] = M::mma(zf[ks], bp[i4][ks], oacc[h][i4]);
                         }
                     }
-                    const int col = col0 + cbase + 16 * h + 4 * g;
+                }
+                // Out of the accumulators a store covers 32 bytes of a row; through LDS (this wave's own
+                // part of the inter-block tile buffer, 64 rows x 32 columns with padded rows) it covers 64.
+                constexpr int OS = 40;  // row stride of the staged tile, elements
+                T* const otile = reinterpret_cast<T*>(Ob + (size_t)w * NH * 4 * 64);
+                // (wavefront-scope fences: the compiler must keep the reads of the inter-block tile above, the
+                // writes of the staged tile and its reads below in this order; LDS itself serves a wave in order)
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+#pragma unroll
+                for (int h = 0; h < NH; ++h)
 #pragma unroll
                     for (int i4 = 0; i4 < 4; ++i4) {
-                        const unsigned tok = (unsigned)(t * 64) + 16 * i4;  // wave-uniform first token of the tile
                         V4 o;
 #pragma unroll
-                        for (int v = 0; v < 4; ++v) o[v] = (T)oacc[i4][v];
-                        const unsigned off = (col < dv && tok + r < nrows) ? (r * ots + col) * (unsigned)sizeof(T) : kOob;
-                        buf_store8(ob, off, tok < nrows ? tok * ots * (unsigned)sizeof(T) : 0u, __builtin_bit_cast(u32x2, o));
+                        for (int v = 0; v < 4; ++v) o[v] = (T)oacc[h][i4][v];
+                        *reinterpret_cast<V4*>(otile + (16 * i4 + r) * OS + 16 * h + 4 * g) = o;
+                    }
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                {
+                    const int orow = lane >> 2, ocol = col0 + cbase + 8 * (lane & 3);
+                    const unsigned tok0 = (unsigned)(t * 64);
+#pragma unroll
+                    for (int p4 = 0; p4 < 4; ++p4) {
+                        const int row = orow + 16 * p4;
+                        const u32x4 val = *reinterpret_cast<const u32x4*>(otile + row * OS + 8 * (lane & 3));
+                        const unsigned tok = tok0 + 16 * p4;  // wave-uniform first token of these 16 rows
+                        const unsigned off = (ocol < colend && tok + orow < nrows) ? (orow * ots + ocol) * (unsigned)sizeof(T) : kOob;
+                        buf_store16(ob, off, tok < nrows ? tok * ots * (unsigned)sizeof(T) : 0u, val);
                     }
                 }
             }

@@ -23,22 +23,29 @@
 
 namespace la {
 
-constexpr int kNgThreads = 256;
+// Threads of a workgroup: TPR threads share a row; rows of one or two wavefronts travel four or two to a
+// workgroup of 256, wider rows take a workgroup of 256, 512 or 1024 threads to themselves.
+constexpr int ng_threads(int tpr) { return tpr >= 256 ? tpr : 256; }
 
-// both sums over the TPR threads of a row at once
+// both sums over the TPR threads of a row at once (every thread of the workgroup takes part)
 template <int TPR>
 __device__ __forceinline__ void row_sum2(float& a, float& b, float* red) {
-    if (TPR == 256) {
+    if (TPR >= 128) {
+        constexpr int NWV = TPR / 64;  // wavefronts per row
         a = wave_sum(a);
         b = wave_sum(b);
-        const int w = threadIdx.x >> 6;
+        const int w = threadIdx.x >> 6, w0 = w / NWV * NWV;
         if ((threadIdx.x & 63) == 0) {
             red[w] = a;
-            red[4 + w] = b;
+            red[16 + w] = b;
         }
         __syncthreads();
-        a = red[0] + red[1] + red[2] + red[3];
-        b = red[4] + red[5] + red[6] + red[7];
+        a = b = 0.f;
+#pragma unroll
+        for (int i = 0; i < NWV; ++i) {
+            a += red[w0 + i];
+            b += red[16 + w0 + i];
+        }
         __syncthreads();
         return;
     }
@@ -56,13 +63,13 @@ __device__ __forceinline__ float sigmoidf(float x) {
 }
 
 template <typename T, int NV, int TPR>
-__global__ __launch_bounds__(kNgThreads) void norm_gate_fwd_kernel(const T* __restrict__ o, const T* __restrict__ g,
+__global__ __launch_bounds__(ng_threads(TPR)) void norm_gate_fwd_kernel(const T* __restrict__ o, const T* __restrict__ g,
                                                                   const T* __restrict__ w, const T* __restrict__ b,
                                                                   T* __restrict__ y, float* __restrict__ mean,
                                                                   float* __restrict__ rstd, int64_t rows, int cols, float eps) {
     constexpr int E = Pack16<T>::N;
-    constexpr int RPG = kNgThreads / TPR;  // rows a workgroup holds at a time
-    __shared__ float red[8];
+    constexpr int RPG = ng_threads(TPR) / TPR;  // rows a workgroup holds at a time
+    __shared__ float red[32];
     const int l = threadIdx.x % TPR;
     const float inv = 1.0f / (float)cols;
     for (int64_t row0 = (int64_t)blockIdx.x * RPG; row0 < rows; row0 += (int64_t)gridDim.x * RPG) {
@@ -135,16 +142,16 @@ __global__ __launch_bounds__(kNgThreads) void norm_gate_fwd_kernel(const T* __re
 
 // `part`: gridDim.x rows of [d weight | d bias] partial column sums, 2 * cols floats each.
 template <typename T, int NV, int TPR>
-__global__ __launch_bounds__(kNgThreads) void norm_gate_bwd_kernel(const T* __restrict__ o, const T* __restrict__ g,
+__global__ __launch_bounds__(ng_threads(TPR)) void norm_gate_bwd_kernel(const T* __restrict__ o, const T* __restrict__ g,
                                                                   const T* __restrict__ w, const T* __restrict__ b,
                                                                   const float* __restrict__ mean, const float* __restrict__ rstd,
                                                                   const T* __restrict__ dy, T* __restrict__ d_o,
                                                                   T* __restrict__ d_g, float* __restrict__ part,
                                                                   int64_t rows, int cols) {
     constexpr int E = Pack16<T>::N;
-    constexpr int RPG = kNgThreads / TPR;
-    __shared__ float red[8];
-    __shared__ float comb[RPG > 1 ? 3 * 64 * NV * E * 2 : 1];  // partial sums of waves 1..3 (TPR = 64)
+    constexpr int RPG = ng_threads(TPR) / TPR;
+    __shared__ float red[32];
+    __shared__ float comb[RPG > 1 ? (RPG - 1) * TPR * NV * E * 2 : 1];  // column sums of the rows beside the first
     const int l = threadIdx.x % TPR;
     float wf[NV][E], bf[NV][E];  // this thread's columns of weight and bias
     float aw[NV][E], ab[NV][E];  // ... and of the column sums
@@ -218,29 +225,29 @@ __global__ __launch_bounds__(kNgThreads) void norm_gate_bwd_kernel(const T* __re
             }
         }
     }
-    // column sums of this workgroup: with one wavefront per row, the four wavefronts hold the same
-    // columns and are added up in wave order first
+    // column sums of this workgroup: the thread groups of its rows hold the same columns and are
+    // added up in row order first
     if (RPG > 1) {
-        const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
-        if (wv > 0) {
+        const int grp = threadIdx.x / TPR;
+        if (grp > 0) {
 #pragma unroll
             for (int u = 0; u < NV; ++u)
 #pragma unroll
                 for (int t = 0; t < E; ++t) {
-                    comb[(((wv - 1) * NV + u) * E + t) * 128 + lane] = aw[u][t];
-                    comb[(((wv - 1) * NV + u) * E + t) * 128 + 64 + lane] = ab[u][t];
+                    comb[((((grp - 1) * NV + u) * E + t) * 2 + 0) * TPR + l] = aw[u][t];
+                    comb[((((grp - 1) * NV + u) * E + t) * 2 + 1) * TPR + l] = ab[u][t];
                 }
         }
         __syncthreads();
-        if (wv > 0) return;
+        if (grp > 0) return;
 #pragma unroll
-        for (int k = 0; k < 3; ++k)
+        for (int k = 0; k < RPG - 1; ++k)
 #pragma unroll
             for (int u = 0; u < NV; ++u)
 #pragma unroll
                 for (int t = 0; t < E; ++t) {
-                    aw[u][t] += comb[((k * NV + u) * E + t) * 128 + lane];
-                    ab[u][t] += comb[((k * NV + u) * E + t) * 128 + 64 + lane];
+                    aw[u][t] += comb[(((k * NV + u) * E + t) * 2 + 0) * TPR + l];
+                    ab[u][t] += comb[(((k * NV + u) * E + t) * 2 + 1) * TPR + l];
                 }
     }
     float* prow = part + (size_t)blockIdx.x * 2 * cols;
@@ -305,8 +312,14 @@ __global__ __launch_bounds__(kRedCols * kRedGroups) void norm_gate_reduce_kernel
 // kernel carries weight, bias and two column sums per column and spreads rows over the workgroup earlier.
 static void ng_shape(int64_t chunks, bool backward, int* tpr, int* nv) {
     *nv = 0;
-    const int64_t wave_max = backward ? 64 : 64 * 4;
-    if (chunks <= wave_max) {
+    if (backward) {
+        // one chunk per thread: the kernel keeps ~7 floats per element of a thread's columns
+        if (chunks > 1024) return;
+        *nv = 1;
+        *tpr = chunks <= 64 ? 64 : chunks <= 128 ? 128 : chunks <= 256 ? 256 : chunks <= 512 ? 512 : 1024;
+        return;
+    }
+    if (chunks <= 64 * 4) {
         *tpr = 64;
         *nv = 1;
         while (64 * *nv < chunks) *nv *= 2;
@@ -327,21 +340,29 @@ static int ng_cus() {
 
 // workgroups of a launch: enough to keep every CU's memory pipeline full, never more than row groups
 static int64_t ng_grid(int64_t rows, int tpr, bool backward) {
-    const int64_t rpg = kNgThreads / tpr, groups = (rows + rpg - 1) / rpg, cap = 4 * (int64_t)ng_cus();
+    const int64_t threads = ng_threads(tpr), rpg = threads / tpr, groups = (rows + rpg - 1) / rpg;
     if (!backward) return groups;  // nothing is carried from row to row: one group of rows per workgroup
+    const int64_t cap = 4 * (int64_t)ng_cus() * 256 / threads;  // ~16 wavefronts per CU
     return groups < cap ? groups : cap;
 }
 
-#define LA_NG_GO(KERNEL, NV, TPR, ...) hipLaunchKernelGGL((KERNEL<T, NV, TPR>), grid, dim3(kNgThreads), 0, st, __VA_ARGS__)
-#define LA_NG_DISPATCH(KERNEL, ...)                                   \
+#define LA_NG_GO(KERNEL, NV, TPR, ...) hipLaunchKernelGGL((KERNEL<T, NV, TPR>), grid, dim3(ng_threads(TPR)), 0, st, __VA_ARGS__)
+#define LA_NG_DISPATCH_FWD(KERNEL, ...)                               \
     do {                                                              \
         if (tpr == 64 && nv == 1) LA_NG_GO(KERNEL, 1, 64, __VA_ARGS__);       \
         else if (tpr == 64 && nv == 2) LA_NG_GO(KERNEL, 2, 64, __VA_ARGS__);  \
-        else if (tpr == 64 && nv == 4) LA_NG_GO(KERNEL, 4, 64, __VA_ARGS__);  \
-        else if (tpr == 64) LA_NG_GO(KERNEL, 8, 64, __VA_ARGS__);             \
+        else if (tpr == 64) LA_NG_GO(KERNEL, 4, 64, __VA_ARGS__);             \
         else if (nv == 1) LA_NG_GO(KERNEL, 1, 256, __VA_ARGS__);              \
         else if (nv == 2) LA_NG_GO(KERNEL, 2, 256, __VA_ARGS__);              \
         else LA_NG_GO(KERNEL, 4, 256, __VA_ARGS__);                           \
+    } while (0)
+#define LA_NG_DISPATCH_BWD(KERNEL, ...)                               \
+    do {                                                              \
+        if (tpr == 64) LA_NG_GO(KERNEL, 1, 64, __VA_ARGS__);          \
+        else if (tpr == 128) LA_NG_GO(KERNEL, 1, 128, __VA_ARGS__);   \
+        else if (tpr == 256) LA_NG_GO(KERNEL, 1, 256, __VA_ARGS__);   \
+        else if (tpr == 512) LA_NG_GO(KERNEL, 1, 512, __VA_ARGS__);   \
+        else LA_NG_GO(KERNEL, 1, 1024, __VA_ARGS__);                  \
     } while (0)
 
 template <typename T>
@@ -351,7 +372,7 @@ static int ng_fwd(const void* o, const void* g, const void* w, const void* b, vo
     ng_shape(cols / (16 / (int64_t)sizeof(T)), false, &tpr, &nv);
     if (!nv) return LA_E_UNSUPPORTED;
     const dim3 grid((unsigned)ng_grid(rows, tpr, false));
-    LA_NG_DISPATCH(norm_gate_fwd_kernel, static_cast<const T*>(o), static_cast<const T*>(g), static_cast<const T*>(w),
+    LA_NG_DISPATCH_FWD(norm_gate_fwd_kernel, static_cast<const T*>(o), static_cast<const T*>(g), static_cast<const T*>(w),
                    static_cast<const T*>(b), static_cast<T*>(y), mean, rstd, rows, (int)cols, eps);
     return (int)hipGetLastError();
 }
@@ -364,7 +385,7 @@ static int ng_bwd(const void* o, const void* g, const void* w, const void* b, co
     ng_shape(cols / (16 / (int64_t)sizeof(T)), true, &tpr, &nv);
     if (!nv) return LA_E_UNSUPPORTED;
     const dim3 grid((unsigned)ng_grid(rows, tpr, true));
-    LA_NG_DISPATCH(norm_gate_bwd_kernel, static_cast<const T*>(o), static_cast<const T*>(g), static_cast<const T*>(w),
+    LA_NG_DISPATCH_BWD(norm_gate_bwd_kernel, static_cast<const T*>(o), static_cast<const T*>(g), static_cast<const T*>(w),
                    static_cast<const T*>(b), mean, rstd, static_cast<const T*>(dy), static_cast<T*>(d_o), static_cast<T*>(d_g),
                    part, rows, (int)cols);
     int rc = (int)hipGetLastError();
@@ -374,7 +395,8 @@ static int ng_bwd(const void* o, const void* g, const void* w, const void* b, co
                        static_cast<T*>(dbias));
     return (int)hipGetLastError();
 }
-#undef LA_NG_DISPATCH
+#undef LA_NG_DISPATCH_FWD
+#undef LA_NG_DISPATCH_BWD
 #undef LA_NG_GO
 
 static int ng_check(int64_t rows, int64_t cols, int dtype) {
