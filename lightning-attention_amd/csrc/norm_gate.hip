@@ -5,14 +5,15 @@
 // (tokens, embed_dim) tensors forward and eleven backward; here three and five).
 //
 // Same data movement as the SimpleRMSNorm kernels: a row of o, g (and dy) is read once with 16-byte
-// non-temporal loads into registers, reduced, and the results written once.  Workgroups have 256 threads;
-// a row belongs to one wavefront (TPR = 64, four rows per workgroup at a time) or to the whole
-// workgroup (TPR = 256).  The forward kernel takes one group of rows per workgroup and fetches weight and
-// bias from the caches.  The backward kernel walks the rows with a grid stride: a thread always holds
-// the same columns, so weight and bias stay in registers as floats and the column sums (d weight,
-// d bias) are accumulated in registers over all rows a thread sees.  Those partial sums go to a scratch
-// buffer, one row per workgroup, and a second small kernel adds them up in a fixed order: deterministic,
-// no atomics.
+// non-temporal loads into registers, reduced, and the results written once.  TPR threads share a row:
+// one or two wavefronts (four or two rows to a workgroup of 256 threads) or a whole workgroup of 256,
+// 512 or 1024 threads.  The forward kernel takes one group of rows per workgroup and fetches weight and
+// bias from the caches.  The backward kernel walks the rows with a grid stride and gives every thread one
+// 16-byte chunk of the row: a thread always holds the same columns, so weight and bias stay in registers
+// as floats and the column sums (d weight, d bias) are accumulated in registers over all rows a thread
+// sees (118 registers: four waves per SIMD; with more chunks per thread it ran at two).  Those partial
+// sums go to a scratch buffer, one row per workgroup, and a second small kernel adds them up in a fixed
+// order: deterministic, no atomics.
 //
 // Per element, float32 throughout:
 //   forward   xh = (o - mean) rstd ; ln = xh w + b ; sg = 1 / (1 + exp(-g)) ; y = ln sg
