@@ -13,11 +13,12 @@ measurement in milliseconds: W untimed warm-up steps, then exactly K steps betwe
 device synchronisations on the host clock.  The same K steps are also bracketed one by
 one with HIP events (``step_event_ms``: median, min, mean).
 
-The secondary measurements (fwd / bwd split, n sweep, other configurations, SRMSNorm,
-per-launch roofline figures) run BEFORE the headline region, so that the chip has been
-under load for a while when it starts: coming out of idle its power management takes
-some 25 steps to settle (the first steps run fast, the next ones up to 40 % slow), which
-``from_idle`` records with the same W / K protocol at the very start of the run.
+The secondary measurements (fwd / bwd split, n sweep, other configurations, SRMSNorm and,
+last, the per-launch roofline figures of the step's own kernels) run BEFORE the headline
+region, so that the chip has been under this load for a while when it starts: coming out of
+idle, or after a change of workload, its power management takes some 25 steps to settle (the
+first steps run fast, the next ones up to 40 % slow), which ``from_idle`` records with the
+same W / K protocol at the very start of the run.
 The CPU baselines (the oracle's naive paths on the host cores, bounded samples) come last.
 """
 import argparse
@@ -303,58 +304,6 @@ def main():
     out = {}
     st = torch.cuda.current_stream().cuda_stream
 
-    # ---- per-launch figures: direct calls of the C entry points, HIP events on the launch stream ----
-    counters = counter_traffic()
-    buf = [torch.empty_like(v) for _ in range(3)]
-    qd, kd, vd = q.detach(), k.detach(), v.detach()
-
-    def fwd_launch():  # O = sweep(Q, K, V)
-        rc = L.la_fwd(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), s.data_ptr(), buf[0].data_ptr(), B, H, N, D, D, 0, None, 0, st)
-        assert rc == 0, rc
-
-    def dq_launch():  # dQ = sweep(dO, V, K): the same kernel instantiation on other operands
-        rc = L.la_fwd(do.data_ptr(), vd.data_ptr(), kd.data_ptr(), s.data_ptr(), buf[0].data_ptr(), B, H, N, D, D, 0, None, 0, st)
-        assert rc == 0, rc
-
-    def bwd_launches():  # dQ, then dK and dV in one launch
-        rc = L.la_bwd(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), s.data_ptr(), do.data_ptr(), buf[0].data_ptr(),
-                      buf[1].data_ptr(), buf[2].data_ptr(), B, H, N, D, D, 0, None, 0, st)
-        assert rc == 0, rc
-
-    def launch_entry(kernel, what, ts, nbytes, nflop, counter_key):
-        med = statistics.median(ts)
-        c = counters.get(counter_key) or {}
-        return {
-            "kernel": kernel, "launch": what, "bound": "hbm",
-            "achieved": round(nbytes / (med * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-            "frac": round(nbytes / (med * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-            # HBM bytes per launch: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each scaled by what the
-            # counter reads for a cast kernel of known size (profiles/, written by benchmarks/profile_summary.py)
-            "traffic": c.get("hbm_bytes"),
-            "traffic_source": ("profiles/%s" % os.path.basename(TRAFFIC_JSON)) if c else None,
-            "algorithmic_bytes": nbytes, "launch_ms": stats(ts),
-            "mfma_tflops": round(nflop / (med * 1e-3) / 1e12, 1),
-            "mfma_frac": round(nflop / (med * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
-        }
-
-    fwd_ts = event_times(fwd_launch, 40, warm=10)
-    dq_ts = event_times(dq_launch, 40, warm=5)
-    bwd_ts = event_times(bwd_launches, 40, warm=5)
-    pair_ts = [max(b_ - statistics.median(dq_ts), 1e-6) for b_ in bwd_ts]
-    fb, ff = bytes_per_token(D, D, "fwd") * tokens, flops_per_token(D, D, "fwd") * tokens
-    pair_bytes = 6 * D * 2 * tokens  # q, k, v, dO read once; dK, dV written once
-    pair_flop = flops_per_token(D, D, "bwd") * tokens - ff
-    roofline = launch_entry("la_sweep_pipe_kernel<bf16, DKP=128, 64 columns, forward, decay>",
-                            "O = sweep(Q,K,V); a step is this, the same for dQ, and one launch for dK + dV",
-                            fwd_ts, fb, ff, "forward")
-    other_launches = [
-        launch_entry("la_sweep_pipe_kernel<bf16, DKP=128, 64 columns, forward, decay>", "dQ = sweep(dO,V,K)", dq_ts, fb, ff, "forward"),
-        launch_entry("la_sweep_pipe_kernel<bf16, DKP=128, 128 columns, reverse, decay>",
-                     "dK + dV in one launch (la_bwd minus the dQ launch, gap between the two included)",
-                     pair_ts, pair_bytes, pair_flop, "reverse_pair"),
-    ]
-    buf = None
-
     if not args.no_sweep:
         # fwd / bwd split at the metric shape (events, reference protocol: bwd = o.backward(do, retain_graph))
         o = lightning_attn_func(q, k, v, s)
@@ -439,10 +388,62 @@ def main():
         }
         del x, dy, y
 
-    # ---- the headline region -------------------------------------------------------------------------
     if q is None or q.shape != (B, H, N, D):
         q = k = v = do = None
         q, k, v, do = inputs(N)
+    # ---- per-launch figures: direct calls of the C entry points, HIP events on the launch stream ----
+    counters = counter_traffic()
+    buf = [torch.empty_like(v) for _ in range(3)]
+    qd, kd, vd = q.detach(), k.detach(), v.detach()
+
+    def fwd_launch():  # O = sweep(Q, K, V)
+        rc = L.la_fwd(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), s.data_ptr(), buf[0].data_ptr(), B, H, N, D, D, 0, None, 0, st)
+        assert rc == 0, rc
+
+    def dq_launch():  # dQ = sweep(dO, V, K): the same kernel instantiation on other operands
+        rc = L.la_fwd(do.data_ptr(), vd.data_ptr(), kd.data_ptr(), s.data_ptr(), buf[0].data_ptr(), B, H, N, D, D, 0, None, 0, st)
+        assert rc == 0, rc
+
+    def bwd_launches():  # dQ, then dK and dV in one launch
+        rc = L.la_bwd(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), s.data_ptr(), do.data_ptr(), buf[0].data_ptr(),
+                      buf[1].data_ptr(), buf[2].data_ptr(), B, H, N, D, D, 0, None, 0, st)
+        assert rc == 0, rc
+
+    def launch_entry(kernel, what, ts, nbytes, nflop, counter_key):
+        med = statistics.median(ts)
+        c = counters.get(counter_key) or {}
+        return {
+            "kernel": kernel, "launch": what, "bound": "hbm",
+            "achieved": round(nbytes / (med * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": round(nbytes / (med * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+            # HBM bytes per launch: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each scaled by what the
+            # counter reads for a cast kernel of known size (profiles/, written by benchmarks/profile_summary.py)
+            "traffic": c.get("hbm_bytes"),
+            "traffic_source": ("profiles/%s" % os.path.basename(TRAFFIC_JSON)) if c else None,
+            "algorithmic_bytes": nbytes, "launch_ms": stats(ts),
+            "mfma_tflops": round(nflop / (med * 1e-3) / 1e12, 1),
+            "mfma_frac": round(nflop / (med * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
+        }
+
+    fwd_ts = event_times_timed(fwd_launch)
+    dq_ts = event_times_timed(dq_launch)
+    bwd_ts = event_times_timed(bwd_launches)
+    pair_ts = [max(b_ - statistics.median(dq_ts), 1e-6) for b_ in bwd_ts]
+    fb, ff = bytes_per_token(D, D, "fwd") * tokens, flops_per_token(D, D, "fwd") * tokens
+    pair_bytes = 6 * D * 2 * tokens  # q, k, v, dO read once; dK, dV written once
+    pair_flop = flops_per_token(D, D, "bwd") * tokens - ff
+    roofline = launch_entry("la_sweep_pipe_kernel<bf16, DKP=128, 64 columns, forward, decay>",
+                            "O = sweep(Q,K,V); a step is this, the same for dQ, and one launch for dK + dV",
+                            fwd_ts, fb, ff, "forward")
+    other_launches = [
+        launch_entry("la_sweep_pipe_kernel<bf16, DKP=128, 64 columns, forward, decay>", "dQ = sweep(dO,V,K)", dq_ts, fb, ff, "forward"),
+        launch_entry("la_sweep_pipe_kernel<bf16, DKP=128, 128 columns, reverse, decay>",
+                     "dK + dV in one launch (la_bwd minus the dQ launch, gap between the two included)",
+                     pair_ts, pair_bytes, pair_flop, "reverse_pair"),
+    ]
+    buf = None
+
+    # ---- the headline region -------------------------------------------------------------------------
     ms, ev_ts = timed_steps(step, args.warmup, args.steps)
     tflops = flop_step / (ms * 1e-3) / 1e12
     del q, k, v, do
