@@ -44,7 +44,11 @@ def _in_place_ok(t):
 
 
 def _usable(t):
-    return t if (t.is_contiguous() or _in_place_ok(t)) else t.contiguous()
+    """`t` itself where the kernels can address it, else a dense, 16-byte aligned copy."""
+    if t.is_contiguous():
+        # (a dense view into a larger buffer may start off the 16-byte grid)
+        return t if t.data_ptr() % 16 == 0 else t.clone(memory_format=torch.contiguous_format)
+    return t if _in_place_ok(t) else t.contiguous()
 
 
 def _strides(*tensors):

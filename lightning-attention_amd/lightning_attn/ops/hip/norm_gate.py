@@ -16,6 +16,12 @@ def norm_gate_supported(cols, dtype):
     return bool(_lib.lib().norm_gate_supported(cols, code))
 
 
+def _dense(t):
+    """Row-major and 16-byte aligned (a dense view into a larger buffer may start off that grid)."""
+    t = t.contiguous()
+    return t if t.data_ptr() % 16 == 0 else t.clone()
+
+
 class _NormGate(torch.autograd.Function):
     @staticmethod
     def forward(ctx, o, g, weight, bias, eps):
@@ -27,8 +33,8 @@ class _NormGate(torch.autograd.Function):
             raise ValueError("shape mismatch: o %s g %s weight %s bias %s"
                              % (tuple(o.shape), tuple(g.shape), tuple(weight.shape), tuple(bias.shape)))
         code = _lib.dtype_code(o.dtype)
-        o2, g2 = o.reshape(-1, cols).contiguous(), g.reshape(-1, cols).contiguous()
-        weight, bias = weight.contiguous(), bias.contiguous()
+        o2, g2 = _dense(o.reshape(-1, cols)), _dense(g.reshape(-1, cols))
+        weight, bias = _dense(weight), _dense(bias)
         rows = o2.shape[0]
         y = torch.empty_like(o2)
         mean = torch.empty((rows,), dtype=torch.float32, device=o.device)
@@ -48,7 +54,7 @@ class _NormGate(torch.autograd.Function):
         rows, cols = o2.shape
         if dy.device != o2.device:
             raise RuntimeError("norm_gate backward: the upstream gradient is on %s, the inputs on %s" % (dy.device, o2.device))
-        dy2 = dy.to(o2.dtype).reshape(rows, cols).contiguous()
+        dy2 = _dense(dy.to(o2.dtype).reshape(rows, cols))
         code = _lib.dtype_code(o2.dtype)
         d_o, d_g = torch.empty_like(o2), torch.empty_like(g2)
         dw, db = torch.empty_like(weight), torch.empty_like(bias)

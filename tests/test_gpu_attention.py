@@ -602,3 +602,25 @@ def test_many_sequences_at_192_take_the_wide_workgroups(dtype):
     check(got, want, dtype, "many sequences, d = 192")
     for a, c in zip(got, run_hip(q, k, v, s, do, wide=False)):
         assert torch.equal(a, c)
+
+
+def test_dense_views_off_the_16_byte_grid_are_copied():
+    """A contiguous view that starts 8 bytes into a larger buffer: the kernels need 16-byte aligned rows, so the
+    operator works on an aligned copy instead of handing the pointer on (which the C entry points refuse)."""
+    b, h, n, d = 1, 2, 130, 64
+    q, k, v, do = make_inputs(b, h, n, d, d, torch.bfloat16, 0.5, seed=3)
+    s = _build_slope_tensor(h)
+
+    def off_grid(t):
+        buf = torch.empty(t.numel() + 4, dtype=t.dtype, device=DEV)
+        view = buf[4:].view(t.shape)
+        view.copy_(t)
+        assert view.is_contiguous() and view.data_ptr() % 16 == 8
+        return view
+
+    qg, kg, vg = (off_grid(t).requires_grad_() for t in (q, k, v))
+    o = lightning_attn_func(qg, kg, vg, s.to(DEV))
+    o.backward(off_grid(do))
+    torch.cuda.synchronize()
+    want = oracle.linear_attn_fwd_bwd(q, k, v, s, do, torch.float32)
+    check((o.detach(), qg.grad, kg.grad, vg.grad), want, torch.bfloat16, "views off the 16-byte grid")

@@ -94,3 +94,22 @@ def test_norm_gate_argument_checks():
     assert rc == -4
     empty = norm_gate(o[:0], g[:0], w, b)
     assert empty.shape == (0, 64)
+
+
+def test_norm_gate_on_views_off_the_16_byte_grid():
+    o, g, w, b, dy = _inputs((33, 256), torch.bfloat16, seed=8)
+
+    def off_grid(t):
+        buf = torch.empty(t.numel() + 4, dtype=t.dtype, device=DEV)
+        view = buf[4:].view(t.shape)
+        view.copy_(t)
+        assert view.data_ptr() % 16 == 8
+        return view
+
+    leaves = [off_grid(t).requires_grad_() for t in (o, g, w, b)]
+    y = norm_gate(*leaves, 1e-5)
+    y.backward(off_grid(dy))
+    torch.cuda.synchronize()
+    want64 = oracle.norm_gate_fwd_bwd(o, g, w, b, dy, 1e-5, torch.float64)
+    for name, a, r in zip(("y", "d_o", "d_g", "d_weight", "d_bias"), [y.detach()] + [t.grad for t in leaves], want64):
+        assert rel_norm(a, r) < 5e-3, (name, rel_norm(a, r))
