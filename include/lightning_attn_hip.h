@@ -144,6 +144,40 @@ int la_bwd_opts(const void *q, const void *k, const void *v, const float *s, con
                 void *workspace, size_t ws_bytes, const la_launch_opts *opts, void *stream);
 
 /*
+ * Forward and backward pass as a pair: the forward pass leaves its d x e float state K^T V at a few
+ * token boundaries, and the dQ sweep of the backward pass - whose state V^T K is the transpose - starts
+ * one chunk of each sequence at each of them.  It then needs neither warm-up blocks nor collect and scan
+ * launches to run as several workgroups per sequence, which is what lets it use 128-column workgroups
+ * when b*h alone gives the chip one or two workgroups per compute unit (b*h of 65 .. 128 on 256 CUs,
+ * 64 < d <= 128, e <= 128, bf16 / fp16).  The reference recomputes that state in its backward pass
+ * (lightning_attn/ops/triton/lightning_attn2.py:240-280) and saves the inputs only (:432); keeping a few
+ * states as well is a deviation made for speed.  Gradients agree with la_bwd's to rounding (the state is
+ * summed in the same order but its operands are rounded to the tensors' dtype in the other role).
+ *
+ * la_saved_state_bytes: bytes the pair uses for these shapes and options, 0 where it would not help (then
+ * la_fwd_save is la_fwd_opts and la_bwd_saved is la_bwd_opts).  Layout: for each of the b*h sequences
+ * m = bytes / (b*h*d*e*4) row-major d x e float matrices, matrix j being
+ *     sum over tokens t < T of exp(-s[h] (T - t)) k_t^T v_t,   T = (j + 1) * la_saved_state_interval(...).
+ * la_fwd_save: la_fwd_opts that also fills `saved` (16-byte aligned, saved_bytes >= la_saved_state_bytes;
+ * otherwise, and with saved == NULL, nothing is saved).  la_bwd_saved: la_bwd_opts that uses `saved` as left
+ * by la_fwd_save for the same tensors, shapes and options (same conditions; otherwise exactly la_bwd_opts).
+ */
+size_t la_saved_state_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
+                            const la_launch_opts *opts);
+int64_t la_saved_state_interval(int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
+                                const la_launch_opts *opts);
+int la_fwd_save(const void *q, const void *k, const void *v, const float *s, void *o,
+                const int64_t *strides,
+                int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
+                void *workspace, size_t ws_bytes, const la_launch_opts *opts,
+                float *saved, size_t saved_bytes, void *stream);
+int la_bwd_saved(const void *q, const void *k, const void *v, const float *s, const void *dout,
+                 void *dq, void *dk, void *dv, const int64_t *strides,
+                 int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
+                 void *workspace, size_t ws_bytes, const la_launch_opts *opts,
+                 const float *saved, size_t saved_bytes, void *stream);
+
+/*
  * la_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc) and so cannot supply the workspace that makes few
  * long sequences fast: same arguments without the workspace pair, same results bit for bit as la_fwd

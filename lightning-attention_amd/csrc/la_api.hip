@@ -14,6 +14,11 @@ int sweep_fwd_rev_once(const SweepIO& fwd, const SweepIO& rev, const float* s, i
 int sweep2(const SweepIO& io0, const SweepIO& io1, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv,
            int dtype, bool reverse, void* ws, size_t ws_bytes, const Opts& opts, hipStream_t st);
 size_t sweep_workspace_bytes(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int dtype, const Opts& opts);
+SavedPlan plan_saved(int64_t bh, int64_t n, int64_t d, int64_t e, int dtype, const Opts& opts);
+int sweep_saving(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
+                 float* save, int save_len, hipStream_t st);
+int sweep_resumed(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
+                  const float* saved, int nchunk, int chunk_len, hipStream_t st);
 int sweep_f32(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
               int64_t n, int64_t dk, int64_t dv, bool reverse, int chunks, hipStream_t st);
 int sweep_f32_bwd_once(const void* q, const void* k, const void* v, const void* dout, void* dq, void* dk, void* dv,
@@ -84,8 +89,17 @@ static int check_tensor(const Tensor& t, int64_t b, int64_t h, int64_t n, int64_
     return LA_OK;
 }
 
+// States for the backward pass (may be absent): memory the forward pass writes / the backward pass reads.
+struct Saved {
+    float* p;
+    size_t bytes;
+};
+static bool saved_usable(const Saved& sv, const SavedPlan& pl) {
+    return pl.nchunk > 1 && sv.p && sv.bytes >= pl.bytes && al16(sv.p);
+}
+
 static int fwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s, const Tensor& o, int64_t b, int64_t h,
-               int64_t n, int64_t d, int64_t e, int dtype, const Scratch& ws, const Opts& opts, hipStream_t st) {
+               int64_t n, int64_t d, int64_t e, int dtype, const Scratch& ws, const Opts& opts, const Saved& sv, hipStream_t st) {
     int rc = check_dims(b, h, n, d, e, dtype);
     if (rc != LA_OK) return rc;
     if ((rc = check_opts(opts)) != LA_OK) return rc;
@@ -96,12 +110,16 @@ static int fwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s
         if (!ts[i]->p) return LA_E_NULLPTR;
     for (int i = 0; i < 4; ++i)
         if ((rc = check_tensor(*ts[i], b, h, n, cols[i], dtype)) != LA_OK) return rc;
+    if (sv.p) {
+        const SavedPlan pl = plan_saved(b * h, n, d, e, dtype, opts);
+        if (saved_usable(sv, pl)) return sweep_saving(io(q, k, v, o), s, b * h, h, n, d, e, dtype, sv.p, pl.chunk_len, st);
+    }
     return run(q, k, v, o, s, b * h, h, n, d, e, dtype, false, ws, opts, st);
 }
 
 static int bwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s, const Tensor& dout, const Tensor& dq,
                const Tensor& dk, const Tensor& dv, int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
-               const Scratch& ws, const Opts& opts, hipStream_t st) {
+               const Scratch& ws, const Opts& opts, const Saved& sv, hipStream_t st) {
     int rc = check_dims(b, h, n, d, e, dtype);
     if (rc != LA_OK) return rc;
     if ((rc = check_opts(opts)) != LA_OK) return rc;
@@ -133,7 +151,11 @@ static int bwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s
         if (rc == LA_OK) return run(k, q, dout, dv, s, b * h, h, n, d, e, dtype, true, ws, opts, st);
         if (rc != LA_E_UNSUPPORTED) return rc;
     }
-    rc = run(dout, v, k, dq, s, b * h, h, n, e, d, dtype, false, ws, opts, st);
+    const SavedPlan pl = sv.p ? plan_saved(b * h, n, d, e, dtype, opts) : SavedPlan{1, 0, 0};
+    if (saved_usable(sv, pl))  // the chunks of dQ start from the states the forward pass left
+        rc = sweep_resumed(io(dout, v, k, dq), s, b * h, h, n, e, d, dtype, sv.p, pl.nchunk, pl.chunk_len, st);
+    else
+        rc = run(dout, v, k, dq, s, b * h, h, n, e, d, dtype, false, ws, opts, st);
     if (rc != LA_OK) return rc;
     // dK_j = sum_{i>=j} lam^(i-j) (v_j . dO_i) q_i   and   dV_j = sum_{i>=j} lam^(i-j) (k_j . q_i) dO_i
     // have the same shape when d == e: one launch, in which they share the reads of dO and q
@@ -189,34 +211,64 @@ extern "C" size_t la_workspace_bytes(int which, int64_t b, int64_t h, int64_t n,
     return la_workspace_bytes_opts(which, b, h, n, d, e, dtype, nullptr);
 }
 
-extern "C" int la_fwd_opts(const void* q, const void* k, const void* v, const float* s, void* o, const int64_t* strides,
+extern "C" int la_fwd_save(const void* q, const void* k, const void* v, const float* s, void* o, const int64_t* strides,
                            int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype, void* workspace,
-                           size_t ws_bytes, const la_launch_opts* opts, void* stream) {
+                           size_t ws_bytes, const la_launch_opts* opts, float* saved, size_t saved_bytes, void* stream) {
     const la::Scratch ws = {workspace, workspace ? ws_bytes : 0};
+    const la::Saved sv = {saved, saved ? saved_bytes : 0};
     const la::Opts& op = opts ? *opts : la::kAuto;
     const hipStream_t st = static_cast<hipStream_t>(stream);
     using la::dense;
     using la::strided;
     if (!strides)
-        return la::fwd(dense(q, h, n, d), dense(k, h, n, d), dense(v, h, n, e), s, dense(o, h, n, e), b, h, n, d, e, dtype, ws, op, st);
+        return la::fwd(dense(q, h, n, d), dense(k, h, n, d), dense(v, h, n, e), s, dense(o, h, n, e), b, h, n, d, e, dtype, ws, op, sv, st);
     return la::fwd(strided(q, strides), strided(k, strides + 3), strided(v, strides + 6), s, strided(o, strides + 9), b, h, n,
-                   d, e, dtype, ws, op, st);
+                   d, e, dtype, ws, op, sv, st);
 }
 
-extern "C" int la_bwd_opts(const void* q, const void* k, const void* v, const float* s, const void* dout, void* dq,
-                           void* dk, void* dv, const int64_t* strides, int64_t b, int64_t h, int64_t n, int64_t d,
-                           int64_t e, int dtype, void* workspace, size_t ws_bytes, const la_launch_opts* opts, void* stream) {
+extern "C" int la_fwd_opts(const void* q, const void* k, const void* v, const float* s, void* o, const int64_t* strides,
+                           int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype, void* workspace,
+                           size_t ws_bytes, const la_launch_opts* opts, void* stream) {
+    return la_fwd_save(q, k, v, s, o, strides, b, h, n, d, e, dtype, workspace, ws_bytes, opts, nullptr, 0, stream);
+}
+
+extern "C" size_t la_saved_state_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
+                                       const la_launch_opts* opts) {
+    const la::Opts& o = opts ? *opts : la::kAuto;
+    if (b <= 0 || n <= 0 || la::check_dims(b, h, n, d, e, dtype) != LA_OK || la::check_opts(o) != LA_OK) return 0;
+    return la::plan_saved(b * h, n, d, e, dtype, o).bytes;
+}
+
+extern "C" int64_t la_saved_state_interval(int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
+                                           const la_launch_opts* opts) {
+    const la::Opts& o = opts ? *opts : la::kAuto;
+    if (b <= 0 || n <= 0 || la::check_dims(b, h, n, d, e, dtype) != LA_OK || la::check_opts(o) != LA_OK) return 0;
+    const la::SavedPlan pl = la::plan_saved(b * h, n, d, e, dtype, o);
+    return pl.nchunk > 1 ? (int64_t)pl.chunk_len * 64 : 0;
+}
+
+extern "C" int la_bwd_saved(const void* q, const void* k, const void* v, const float* s, const void* dout, void* dq,
+                            void* dk, void* dv, const int64_t* strides, int64_t b, int64_t h, int64_t n, int64_t d,
+                            int64_t e, int dtype, void* workspace, size_t ws_bytes, const la_launch_opts* opts,
+                            const float* saved, size_t saved_bytes, void* stream) {
     const la::Scratch ws = {workspace, workspace ? ws_bytes : 0};
+    const la::Saved sv = {const_cast<float*>(saved), saved ? saved_bytes : 0};
     const la::Opts& op = opts ? *opts : la::kAuto;
     const hipStream_t st = static_cast<hipStream_t>(stream);
     using la::dense;
     using la::strided;
     if (!strides)
         return la::bwd(dense(q, h, n, d), dense(k, h, n, d), dense(v, h, n, e), s, dense(dout, h, n, e), dense(dq, h, n, d),
-                       dense(dk, h, n, d), dense(dv, h, n, e), b, h, n, d, e, dtype, ws, op, st);
+                       dense(dk, h, n, d), dense(dv, h, n, e), b, h, n, d, e, dtype, ws, op, sv, st);
     return la::bwd(strided(q, strides), strided(k, strides + 3), strided(v, strides + 6), s, strided(dout, strides + 9),
                    strided(dq, strides + 12), strided(dk, strides + 15), strided(dv, strides + 18), b, h, n, d, e, dtype, ws,
-                   op, st);
+                   op, sv, st);
+}
+
+extern "C" int la_bwd_opts(const void* q, const void* k, const void* v, const float* s, const void* dout, void* dq,
+                           void* dk, void* dv, const int64_t* strides, int64_t b, int64_t h, int64_t n, int64_t d,
+                           int64_t e, int dtype, void* workspace, size_t ws_bytes, const la_launch_opts* opts, void* stream) {
+    return la_bwd_saved(q, k, v, s, dout, dq, dk, dv, strides, b, h, n, d, e, dtype, workspace, ws_bytes, opts, nullptr, 0, stream);
 }
 
 extern "C" int la_fwd(const void* q, const void* k, const void* v, const float* s, void* o, int64_t b, int64_t h,

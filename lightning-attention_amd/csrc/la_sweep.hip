@@ -752,6 +752,80 @@ int sweep(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, i
     return launch_planned(p, bh, n, dk, dv, dtype, reverse, ws, ws_bytes, opts, st);
 }
 
+// States a forward sweep can leave behind for the sweep that follows it over the same tensors in swapped roles.
+// O = sweep(q, k, v) carries the state K^T V (d x e); dQ = sweep(dO, v, k) of the backward pass carries V^T K,
+// its transpose.  Where the forward pass walks each sequence in one piece and leaves the state at c - 1
+// equally spaced block boundaries, the dQ sweep can run as c chunks per sequence from those states - no
+// warm-up blocks, no collect and scan launches - and so in 128-column workgroups where 64-column ones
+// would otherwise be needed to give every CU a workgroup (b*h around 128 on a 256-CU chip).
+// nchunk == 1: not for this shape.
+SavedPlan plan_saved(int64_t bh, int64_t n, int64_t d, int64_t e, int dtype, const Opts& opts) {
+    const SavedPlan none = {1, 0, 0};
+    if (dtype != LA_BF16 && dtype != LA_FP16) return none;
+    if (d <= 64 || d > 128 || e > 128) return none;
+    if (opts.chunks != 0 || opts.wide == LA_OPT_ON || opts.scan == LA_OPT_ON) return none;
+    const int64_t nblk = (n + 63) / 64, cus = num_cus(), units8 = (bh + 7) / 8 * 8;
+    // the forward pass as planned: 64-column workgroups, one walk per sequence
+    if (wide_columns(bh, n, d, e, 1, (size_t)-1, opts)) return none;
+    if (plan_scan(bh, n, d, e, 1, false, opts).nchunk > 1) return none;
+    if (warm_up_chunks(units8 * ((e + 63) / 64), nblk) > 1) return none;
+    // dQ: one 128-column workgroup per sequence and chunk
+    int64_t c = cus / units8;
+    if (c > nblk / 4) c = nblk / 4;
+    if (c > 64) c = 64;
+    if (c < 2) return none;
+    SavedPlan pl;
+    pl.chunk_len = (int)((nblk + c - 1) / c);
+    pl.nchunk = (int)((nblk + pl.chunk_len - 1) / pl.chunk_len);
+    if (pl.nchunk < 2) return none;
+    // against what the dQ sweep would take by its own plan
+    const bool wide = wide_columns(bh, n, e, d, 1, (size_t)-1, opts);
+    const ScanPlan own = plan_scan(bh, n, e, d, 1, wide, opts);
+    const double own_us = own.nchunk > 1 ? own.us : warm_up_us(bh, n, e, d, 1, wide);
+    if ((double)pl.chunk_len * block_us(e, true) >= own_us) return none;
+    pl.bytes = (size_t)bh * (size_t)(pl.nchunk - 1) * (size_t)(d * e) * sizeof(float);
+    return pl;
+}
+
+// The forward sweep as sweep() plans it where plan_saved applies, leaving its state every save_len blocks in `save`.
+int sweep_saving(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
+                 float* save, int save_len, hipStream_t st) {
+    SweepPair p;
+    p.nprod = 1;
+    p.a[0] = make_args(io, s, bh, h, n, dk, dv);
+    p.a[0].nchunk = 1;
+    p.a[0].chunk_start[0] = 0;
+    for (int j = 1; j < 9; ++j) p.a[0].chunk_start[j] = (int)((n + 63) / 64);
+    p.a[1] = p.a[0];
+    p.wide = 0;
+    p.mode = kWarmUp;
+    p.chunk_len = 0;
+    p.state = nullptr;
+    p.save = save;
+    p.save_len = save_len;
+    return sweep_pipe(p, dtype, false, st);
+}
+
+// The sweep (x, y, z) -> out in nchunk chunks of chunk_len blocks that start from `saved`: what sweep_saving over
+// (., z, y) left behind (per sequence nchunk - 1 row-major dv x dk matrices).  128-column workgroups.
+int sweep_resumed(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
+                  const float* saved, int nchunk, int chunk_len, hipStream_t st) {
+    if (dk > 128 || dv > 128 || nchunk < 2 || chunk_len < 1) return LA_E_UNSUPPORTED;
+    SweepPair p;
+    p.nprod = 1;
+    p.a[0] = make_args(io, s, bh, h, n, dk, dv);
+    p.a[0].nslice = 1;
+    p.a[0].zw = 128;
+    p.a[0].nchunk = nchunk;
+    for (int j = 0; j < 9; ++j) p.a[0].chunk_start[j] = 0;
+    p.a[1] = p.a[0];
+    p.wide = 1;
+    p.mode = kResume;
+    p.chunk_len = chunk_len;
+    p.state = const_cast<float*>(saved);
+    return sweep_pipe(p, dtype, false, st);
+}
+
 // Two sweeps of the same shape and direction in one launch.
 int sweep2(const SweepIO& io0, const SweepIO& io1, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv,
            int dtype, bool reverse, void* ws, size_t ws_bytes, const Opts& opts, hipStream_t st) {

@@ -110,11 +110,22 @@ struct SweepPair {
     //             from zero, and leaves the state it ends with in `state` (the last chunk has nothing to leave);
     //   kApply    third launch: it starts from `state`, which the scan kernel run in between has turned
     //             into the state at the start of each chunk.
-    // In the two latter modes the chunks are chunk_len blocks long (a[0].chunk_start is not used) and
-    // `state` holds, per (unit, sweep, slice), nchunk - 1 slots of the state waves' accumulators.
+    //   kResume   a single launch: it starts from `state`, which an earlier sweep over the same y and z in
+    //             swapped roles has left behind (`save` below).
+    // In the three latter modes the chunks are chunk_len blocks long (a[0].chunk_start is not used).  kCollect /
+    // kApply: `state` holds, per (unit, sweep, slice), nchunk - 1 slots of the state waves' accumulators.
+    // kResume: per unit nchunk - 1 plain row-major matrices of dv x dk floats, matrix c - 1 being the
+    // transpose of the state chunk c starts from (pipelined kernel, 128-column workgroups, one sweep).
     int mode;
     int chunk_len;
     float* state;
+    // Forward walk in one piece (pipelined kernel, 64-column workgroups): after every save_len blocks but the
+    // last the state is also written to `save`, per unit (number of such boundaries) row-major dk x dv float
+    // matrices.  The sweep (x', y' = z, z' = y) then has exactly the transposed state at those boundaries
+    // and can start chunks there (kResume): the dQ sweep of the backward pass after the forward pass.
+    // nullptr / 0: nothing is saved.
+    float* save = nullptr;
+    int save_len = 0;
 };
 
 // One launch can also carry sweeps of both directions: the whole backward pass when d == e, dQ walking
@@ -149,9 +160,16 @@ inline int allow_lds(K kern, size_t lds, unsigned char (&done)[kMaxDevices]) {
     return 0;
 }
 
+// Where a forward pass leaves states for the backward pass's dQ sweep (la_sweep.hip): chunks of that sweep,
+// their length in blocks (= blocks between two saved states), bytes of float matrices; nchunk == 1: nowhere.
+struct SavedPlan {
+    int nchunk, chunk_len;
+    size_t bytes;
+};
+
 // Launches the single-barrier pipelined kernel (feature dim up to 128); defined in la_sweep_pipe.hip.
 // n, dk, dv, h, bh, nslice and the chunking must agree between the two sweeps of a pair.
-enum { kWarmUp = 0, kCollect = 1, kApply = 2 };
+enum { kWarmUp = 0, kCollect = 1, kApply = 2, kResume = 3 };
 int sweep_pipe(const SweepPair& p, int dtype, bool reverse, hipStream_t st);
 // Floats of one state slot: the feature dim as the kernel pads it (64 or 128 in the pipelined kernel, 192
 // or 256 in the two-barrier one) times the 64 or 128 columns of a workgroup.  Must agree with the

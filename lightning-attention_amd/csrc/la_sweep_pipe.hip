@@ -375,6 +375,28 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
     const unsigned lane_pr = (r * PS + 8 * g) * E;
     const unsigned lane_ow = (r * ZS + cbase + 4 * g) * E;  // out[i = r][cbase + 4 g ..] within 16 rows
 
+    // Forward walk in one piece with `save`: the state after every save_len blocks but the last goes to memory as
+    // a plain dk x dv float matrix (this wave's 16 columns of it; 64-byte runs).  Rare - once per chunk
+    // of the pass that will start from it -, so the addresses are made where they are used and nothing of
+    // this lives in registers across the loop.
+    int64_t next_save = pair.save != nullptr && pair.save_len > 0 && pair.save_len < nblk ? (int64_t)pair.save_len : -1;
+    auto save_state = [&](const int64_t it) __attribute__((always_inline)) {
+        const int64_t nsave = (nblk - 1) / pair.save_len;  // boundaries per unit
+        const int64_t j = (it + 1) / pair.save_len - 1;
+        const unsigned lr = opaque((unsigned)r), lg = opaque((unsigned)g);
+        const int c = col0 + cbase + (int)lr;
+        float* const dst = pair.save + ((size_t)unit * nsave + j) * ((size_t)dk * dv) + c;
+        if (c < dv) {
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int k = 16 * kt + 4 * (int)lg + v;
+                    if (k < dk) dst[(size_t)k * dv] = st[0][kt][v];
+                }
+        }
+    };
+
     // One iteration.  `xr, yr, zr` hold block it+2 on entry and block it+4 on exit.
     auto iteration = [&](auto role, const int64_t it, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4 (&zr)[ZC]) __attribute__((always_inline)) {
         constexpr bool STATE = decltype(role)::value;
@@ -528,6 +550,14 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
+            if constexpr (!REVERSE && NH == 1) {
+                // a boundary the next pass over these tensors may start from: leave the state after block `it`
+                if (it + 1 == next_save) {
+                    save_state(it);
+                    next_save += pair.save_len;
+                    if (next_save >= nblk) next_save = -1;  // the end of the sequence is no boundary
+                }
+            }
         }
         __syncthreads();
     };
@@ -584,6 +614,21 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
                 st[h][kt] = resume ? *reinterpret_cast<const f32x4*>(src + (size_t)(h * KT + kt) * 256) : (f32x4){0.f, 0.f, 0.f, 0.f};
+        if constexpr (!REVERSE && NH == 2) {
+            if (mode == kResume && chunk > 0) {
+                // state[k][c] = saved[c][k]: this lane's four k of a tile are neighbours in row c of the saved matrix
+                const float* const m = pair.state + ((size_t)unit * (nchunk - 1) + (chunk - 1)) * ((size_t)dk * dv);
+#pragma unroll
+                for (int h = 0; h < NH; ++h) {
+                    const int c = col0 + cbase + 16 * h + r;
+#pragma unroll
+                    for (int kt = 0; kt < KT; ++kt) {
+                        const int k = 16 * kt + 4 * g;  // dk is a multiple of 8: a quartet lies inside or outside
+                        if (c < dv && k < dk) st[h][kt] = *reinterpret_cast<const f32x4*>(m + (size_t)c * dk + k);
+                    }
+                }
+            }
+        }
         walk(std::true_type{});
         if (mode == kCollect) {
             float* const dst = slot0 + (size_t)chunk * SF + lane_slot;
@@ -617,7 +662,11 @@ static int launch_one(const SweepPair& pair, hipStream_t st) {
     if (const int e = allow_lds(kern, lds, lds_allowed)) return e;
     const int units8 = (a.bh + 7) / 8 * 8;
     // the state slots the host sized must be the ones this instantiation reads and writes
-    if (pair.mode != kWarmUp && pipe_state_floats(a.dk, pair.wide != 0) != (size_t)4 * NH * (DKP / 16) * 64 * 4) return LA_E_WORKSPACE;
+    if ((pair.mode == kCollect || pair.mode == kApply) && pipe_state_floats(a.dk, pair.wide != 0) != (size_t)4 * NH * (DKP / 16) * 64 * 4)
+        return LA_E_WORKSPACE;
+    // the plain-matrix forms of the state exist in two instantiations only
+    if (pair.mode == kResume && (REVERSE || NH != 2 || pair.nprod != 1)) return LA_E_UNSUPPORTED;
+    if (pair.save && (REVERSE || NH != 1 || pair.nprod != 1 || pair.mode != kWarmUp || a.nchunk != 1)) return LA_E_UNSUPPORTED;
     const unsigned grid = (unsigned)(units8 * a.nslice * a.nchunk * pair.nprod);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, st, pair);
     return (int)hipGetLastError();
@@ -743,6 +792,7 @@ int sweep_pipe(const SweepPair& p, int dtype, bool reverse, hipStream_t st) {
         return launch_any(q, dtype, reverse, st);
     }
     if (!p.state || p.chunk_len < 1) return LA_E_WORKSPACE;
+    if (p.mode == kResume) return launch_any(p, dtype, reverse, st);  // the states are there already
     // three launches: local end states, their scan, the walk proper
     SweepPair q = p;
     q.mode = kCollect;

@@ -18,7 +18,7 @@ _DTYPES = {torch.bfloat16: LA_BF16, torch.float16: LA_FP16, torch.float32: LA_FP
 SYMBOLS = (
     "la_version", "la_error_string", "la_supported", "la_workspace_bytes",
     "la_fwd", "la_bwd", "la_fwd_strided", "la_bwd_strided", "la_workspace_bytes_opts", "la_fwd_opts", "la_bwd_opts",
-    "la_fwd_static",
+    "la_fwd_static", "la_saved_state_bytes", "la_saved_state_interval", "la_fwd_save", "la_bwd_saved",
     "srmsnorm_fwd", "srmsnorm_bwd", "norm_gate_supported", "norm_gate_workspace_bytes", "norm_gate_fwd", "norm_gate_bwd",
 )
 
@@ -52,13 +52,16 @@ def _tri(v):
 
 
 @contextlib.contextmanager
-def launch_opts(chunks=0, scan=None, wide=None, paired=None, once=None):
+def launch_opts(chunks=0, scan=None, wide=None, paired=None, once=None, save_states=True):
     """Within the block, the attention operators called from this thread map their work onto
     launches as told (the backward pass of an operator follows the options its forward ran under): `chunks` sequence chunks (0 = library's choice); `scan`, `wide`, `paired`,
-    `once` = None (library's choice) / False / True.  For measurements and tests; the results do
+    `once` = None (library's choice) / False / True; `save_states` = False: a forward pass that will be
+    differentiated keeps its inputs only, as the reference does, instead of also leaving a few states
+    for its backward pass (la_fwd_save in the header).  For measurements and tests; the results do
     not depend on it beyond rounding (see la_launch_opts in the header)."""
     prev = current_opts()
     _tls.opts = LaunchOpts(int(chunks or 0), _tri(scan), _tri(wide), _tri(paired), _tri(once))
+    _tls.opts.save_states = bool(save_states)
     try:
         yield _tls.opts
     finally:
@@ -103,6 +106,16 @@ def lib():
             L.la_bwd_opts.restype = _int
             L.la_bwd_opts.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
                                       _vp, _sz, _op, _vp]
+            L.la_saved_state_bytes.restype = _sz
+            L.la_saved_state_bytes.argtypes = [_i64, _i64, _i64, _i64, _i64, _int, _op]
+            L.la_saved_state_interval.restype = _i64
+            L.la_saved_state_interval.argtypes = [_i64, _i64, _i64, _i64, _i64, _int, _op]
+            L.la_fwd_save.restype = _int
+            L.la_fwd_save.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _sz, _op,
+                                      _vp, _sz, _vp]
+            L.la_bwd_saved.restype = _int
+            L.la_bwd_saved.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
+                                       _vp, _sz, _op, _vp, _sz, _vp]
             L.la_fwd_static.restype = _int
             L.la_fwd_static.argtypes = [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp]
             L.srmsnorm_fwd.restype = _int
@@ -162,6 +175,20 @@ def workspace_bytes(which, b, h, n, d, e, code, opts):
     got = _ws_cache.get(key)
     if got is None:
         got = lib().la_workspace_bytes_opts(which, b, h, n, d, e, code, ctypes.byref(opts) if opts is not None else None)
+        if len(_ws_cache) > 4096:
+            _ws_cache.clear()
+        _ws_cache[key] = got
+    return got
+
+
+def saved_state_bytes(b, h, n, d, e, code, opts):
+    """la_saved_state_bytes, remembered per shape like workspace_bytes; 0 where `opts` turn the states off."""
+    if opts is not None and not getattr(opts, "save_states", True):
+        return 0
+    key = ("saved", b, h, n, d, e, code, opts.key() if opts is not None else None, torch.cuda.current_device())
+    got = _ws_cache.get(key)
+    if got is None:
+        got = lib().la_saved_state_bytes(b, h, n, d, e, code, ctypes.byref(opts) if opts is not None else None)
         if len(_ws_cache) > 4096:
             _ws_cache.clear()
         _ws_cache[key] = got

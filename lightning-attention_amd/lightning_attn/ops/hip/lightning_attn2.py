@@ -4,7 +4,9 @@ Same names and call conventions as lightning_attn/ops/triton/lightning_attn2.py:
 and lightning_attn2_no_decay.py:367-471: ``lightning_attn2(q, k, v, s)`` and
 ``lightning_attn2_no_decay(q, k, v)`` with q,k (b,h,n,d), v (b,h,n,e), s holding
 h float32 rates; outputs come from torch.empty, kernels go on the current stream,
-and only the inputs are saved for backward.
+and the inputs are saved for backward - plus, for shapes where the library asks for
+them (la_saved_state_bytes in the header), a few float32 states of the forward walk that let
+the dQ sweep of the backward pass start mid-sequence (8 MiB at b4 h32 n8192 d=e=128).
 
 Where the reference copies (``.contiguous()`` on q, k, v, do, lightning_attn2.py:402-405,
 439-442), bf16 / fp16 tensors whose feature dim is contiguous and whose other strides are
@@ -59,7 +61,9 @@ def _strides(*tensors):
     return (ctypes.c_int64 * len(vals))(*vals)
 
 
-def _fwd(q, k, v, s):
+def _fwd(q, k, v, s, for_backward=False):
+    """Runs the forward pass; returns o, the tensors as the kernels used them and - `for_backward`, where the
+    library has a use for them - the states the backward pass starts its dQ chunks from (else None)."""
     _lib.require_same_device("lightning_attn2", q=q, k=k, v=v)
     if not (q.dtype == k.dtype == v.dtype):
         raise TypeError("q, k, v must share a dtype")
@@ -83,13 +87,16 @@ def _fwd(q, k, v, s):
         sp = s.data_ptr() if s is not None else None
         wp = ws.data_ptr() if ws is not None else None
         strides = None if all(t.is_contiguous() for t in (q, k, v, o)) else _strides(q, k, v, o)
-        rc = L.la_fwd_opts(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, o.data_ptr(), strides, b, h, n, d, e, code,
-                           wp, ws_bytes, ctypes.byref(opts) if opts is not None else None, _lib.stream_ptr(q.device))
+        sv_bytes = _lib.saved_state_bytes(b, h, n, d, e, code, opts) if for_backward else 0
+        saved = torch.empty(sv_bytes // 4, dtype=torch.float32, device=q.device) if sv_bytes else None
+        rc = L.la_fwd_save(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, o.data_ptr(), strides, b, h, n, d, e, code,
+                           wp, ws_bytes, ctypes.byref(opts) if opts is not None else None,
+                           saved.data_ptr() if saved is not None else None, sv_bytes, _lib.stream_ptr(q.device))
     _lib.check(rc, "la_fwd")
-    return o, q, k, v, s
+    return o, q, k, v, s, saved
 
 
-def _bwd(q, k, v, s, do, opts=None):
+def _bwd(q, k, v, s, do, opts=None, saved=None):
     b, h, n, d = q.shape
     e = v.shape[-1]
     L = _lib.lib()
@@ -107,9 +114,11 @@ def _bwd(q, k, v, s, do, opts=None):
         wp = ws.data_ptr() if ws is not None else None
         dense = all(t.is_contiguous() for t in (q, k, v, do, dq, dk, dv))
         strides = None if dense else _strides(q, k, v, do, dq, dk, dv)
-        rc = L.la_bwd_opts(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, do.data_ptr(), dq.data_ptr(), dk.data_ptr(),
-                           dv.data_ptr(), strides, b, h, n, d, e, code, wp, ws_bytes,
-                           ctypes.byref(opts) if opts is not None else None, _lib.stream_ptr(q.device))
+        rc = L.la_bwd_saved(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, do.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                            dv.data_ptr(), strides, b, h, n, d, e, code, wp, ws_bytes,
+                            ctypes.byref(opts) if opts is not None else None,
+                            saved.data_ptr() if saved is not None else None, saved.numel() * 4 if saved is not None else 0,
+                            _lib.stream_ptr(q.device))
     _lib.check(rc, "la_bwd")
     return dq, dk, dv
 
@@ -121,16 +130,16 @@ class LightningAttention2(torch.autograd.Function):
     def forward(ctx, q, k, v, s):
         if s is None:
             raise ValueError("lightning_attn2 needs decay rates s; use lightning_attn2_no_decay")
-        o, q, k, v, s = _fwd(q, k, v, s)
-        ctx.save_for_backward(q, k, v, s)
+        o, q, k, v, s, saved = _fwd(q, k, v, s, any(ctx.needs_input_grad[:3]))
+        ctx.save_for_backward(q, k, v, s, saved)
         # autograd runs backward on a thread of its own: the launch options in force now go with the node
         ctx.la_opts = _lib.current_opts()
         return o
 
     @staticmethod
     def backward(ctx, do):
-        q, k, v, s = ctx.saved_tensors
-        dq, dk, dv = _bwd(q, k, v, s, do, ctx.la_opts)
+        q, k, v, s, saved = ctx.saved_tensors
+        dq, dk, dv = _bwd(q, k, v, s, do, ctx.la_opts, saved)
         return dq, dk, dv, None
 
 
@@ -139,15 +148,15 @@ class LightningAttention2NoDecay(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v):
-        o, q, k, v, _ = _fwd(q, k, v, None)
-        ctx.save_for_backward(q, k, v)
+        o, q, k, v, _, saved = _fwd(q, k, v, None, any(ctx.needs_input_grad))
+        ctx.save_for_backward(q, k, v, saved)
         ctx.la_opts = _lib.current_opts()
         return o
 
     @staticmethod
     def backward(ctx, do):
-        q, k, v = ctx.saved_tensors
-        return _bwd(q, k, v, None, do, ctx.la_opts)
+        q, k, v, saved = ctx.saved_tensors
+        return _bwd(q, k, v, None, do, ctx.la_opts, saved)
 
 
 lightning_attn2 = LightningAttention2.apply

@@ -22,6 +22,7 @@ from .linear_attn_oracle import (  # noqa: F401
     linear_attn_fwd_bwd,
     block_recurrence_fwd,
     block_recurrence_bwd,
+    kv_state,
 )
 from .srmsnorm_oracle import srmsnorm, srmsnorm_fwd_bwd, srmsnorm_f64  # noqa: F401
 from .norm_gate_oracle import norm_gate as norm_gate_ref, norm_gate_fwd_bwd, norm_gate_closed_form  # noqa: F401

@@ -21,6 +21,10 @@ What pins each function (see tests/test_oracle_*.py):
   gradient sums evaluated by the C brute force, plus gradcheck in fp64.
 * block_recurrence_* : identity with linear_attn_f64 for ragged n and for
   block sizes 16/64/128, concatenation property, linearity.
+* kv_state : with k, v zeroed from token T on, the naive output at i >= T is
+  exp(-s (i - T)) q_i KV_T (checked against linear_attn_f64 with unit-vector
+  queries, which reads the matrix out row by row); KV_T over a split sequence
+  obeys KV_T = exp(-s (T - T1)) KV_T1 + (state of the tokens T1..T alone).
 
 No function here is "parity unpinned".
 """
@@ -148,6 +152,18 @@ def block_recurrence_fwd(q, k, v, s=None, block=64, dtype=torch.float64):
         out[:, :, sl] = ((Q @ K.transpose(2, 3)) * D) @ V + lq * (Q @ kv)
         kv = lb * kv + (K * lk).transpose(2, 3) @ V
     return out[:, :, :n]
+
+
+def kv_state(k, v, s, T, dtype=torch.float64):
+    """The d x e state the forward recurrence holds after the first T tokens,
+    KV_T = sum_{t<T} exp(-s (T - t)) k_t^T v_t: the `kv` accumulator of
+    lightning_attn2.py:55, 78-84 after T / BLOCK iterations, written as the closed-form sum.
+    k: (b,h,n,d), v: (b,h,n,e) -> (b,h,d,e)."""
+    b, h, n, d = k.shape
+    rate = _lam(s, h, dtype).view(1, h, 1, 1)
+    t = torch.arange(T, dtype=dtype).view(1, 1, T, 1)
+    w = torch.exp(-rate * (T - t))
+    return (k[:, :, :T].to(dtype) * w).transpose(2, 3) @ v[:, :, :T].to(dtype)
 
 
 def block_recurrence_bwd(q, k, v, s, do, block=64, dtype=torch.float64):

@@ -124,3 +124,29 @@ def test_config1_plumbing():
     bq, bk, bv = oracle.block_recurrence_bwd(q, k, v, s, do, 64)
     for a, c in ((o, ob), (dq, bq), (dk, bk), (dv, bv)):
         assert ((a.double() - c).norm() / c.norm()).item() < 1e-5
+
+
+@pytest.mark.parametrize("decay", [True, False])
+def test_kv_state_read_out_by_the_naive_path(decay):
+    """kv_state against the naive path: with k, v zeroed from token T on, o_i = exp(-s (i - T)) q_i KV_T
+    for i >= T; unit-vector queries read KV_T out row by row.  Plus the split rule of the recurrence."""
+    b, h, n, d, e, T = 2, 3, 40, 5, 4, 23
+    _, k, v, _ = _rand(b, h, n, d, e, seed=11)
+    s = oracle.build_slope_tensor(h) if decay else None
+    rate = s.reshape(-1).double() if decay else torch.zeros(h, dtype=torch.float64)
+    S = oracle.kv_state(k, v, s, T)
+    assert S.shape == (b, h, d, e)
+    k0, v0 = k.clone(), v.clone()
+    k0[:, :, T:] = 0
+    v0[:, :, T:] = 0
+    for row in range(d):
+        q = torch.zeros(b, h, n, d, dtype=torch.float64)
+        q[..., row] = 1.0
+        o = oracle.linear_attn_f64(q, k0, v0, s)
+        for i in (T, T + 1, n - 1):
+            want = torch.exp(-rate * (i - T)).view(1, h, 1) * S[:, :, row, :]
+            assert torch.allclose(o[:, :, i, :], want, rtol=1e-12, atol=1e-12)
+    T1 = 9
+    tail = oracle.kv_state(k[:, :, T1:], v[:, :, T1:], s, T - T1)
+    joined = torch.exp(-rate * (T - T1)).view(1, h, 1, 1) * oracle.kv_state(k, v, s, T1) + tail
+    assert torch.allclose(S, joined, rtol=1e-12, atol=1e-12)
