@@ -17,7 +17,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build", "obj")
 OUT_DIR = os.path.join(HERE, "lightning_attn", "_C")
 OUT = os.path.join(OUT_DIR, "liblightning_attn_hip.so")
-SOURCES = ["la_api.hip", "la_sweep.hip", "la_sweep_pipe.hip", "la_sweep_wide.hip", "la_sweep_f32.hip", "srmsnorm.hip", "norm_gate.hip"]
+SOURCES = ["la_api.hip", "la_sweep.hip", "la_sweep_pipe.hip", "la_sweep_pipe_split.hip", "la_sweep_f32.hip", "srmsnorm.hip", "norm_gate.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -1,6 +1,6 @@
-// Single-sweep decayed linear attention for gfx950 (bf16 / fp16 MFMA, fp32 state).
+// Decayed linear attention as directional "sweeps", and how a sweep is mapped onto kernel launches (host side).
 //
-// One generic "sweep" computes, per (batch, head),
+// One generic sweep computes, per (batch, head),
 //     forward  direction:  out_i = sum_{j<=i} lam^(i-j) (x_i . y_j) z_j
 //     reverse  direction:  out_i = sum_{j>=i} lam^(j-i) (x_i . y_j) z_j
 // with lam = exp(-s_h).  The four products of the operator are instances of it:
@@ -8,525 +8,29 @@
 //     dK = sweep_rev(V , dO, Q )      dV = sweep_rev(K , Q , dO)
 // (lightning_attn/ops/triton/lightning_attn2.py:8-85 forward, :88-395 backward.)
 //
-// The sequence is cut into blocks of 64 tokens.  A workgroup of 8 wavefronts owns
-// one (batch, head, 64-column slice of z/out) and walks the blocks in order.  The
-// wavefronts are specialised so that every SIMD holds two waves with different
-// instruction mixes:
-//   waves 0-3 ("score" waves)   S^T = y x^T tiles -> decay/mask -> P (LDS);
-//                               out^T = inter + z^T P^T ; store out
-//   waves 4-7 ("state" waves)   own the dk x 16 column slab of the state
-//                               S = sum lam^.. y_j^T z_j in fp32 accumulators;
-//                               inter = Lout * (state^T x^T) -> LDS;
-//                               state = lam^64 state + y^T (z * Lupd)
-// State and z^T fragments never leave registers: the accumulator layout of one
-// MFMA is reused as the A operand of the next with a matching permutation of the
-// contraction index on the B side.  Transposed operands (y^T, z^T) come from the
-// LDS transpose read ds_read_b64_tr_b16.  x/y/z tiles are double-buffered in LDS
-// (global -> registers one block ahead -> LDS), two barriers per block.
+// The kernel is the pipelined one of la_sweep_pipe_body.h for every feature dim up to 256.  This file
+// decides, from the shape and the compute units of the device, how many columns of z / out a workgroup
+// takes (64 or 128), whether a long walk over few sequences is cut into chunks (from warm-up blocks, or
+// from scanned states in a workspace), and which sweeps of a backward pass share a launch.
 #include "la_sweep_common.h"
 #include "lightning_attn_hip.h"
 
 namespace la {
 
-template <int DKP>
-struct SweepLds {
-#ifndef LA_XPAD
-#define LA_XPAD 16
-#endif
-#ifndef LA_ZPAD
-#define LA_ZPAD 8
-#endif
-    static constexpr int XS = DKP + LA_XPAD;  // row stride (elements) of the x / y tiles
-    static constexpr int ZS = 64 + LA_ZPAD;   // row stride of the z slice and the P tile
-    static constexpr int NBUF = DKP <= 192 ? 2 : 1;
-    static constexpr int TILE = 2 * 64 * XS + 64 * ZS;  // elements of one x+y+z buffer
-    static constexpr size_t bytes(size_t elt) { return (size_t)(NBUF * TILE + 64 * ZS) * elt + 4 * 4 * 64 * 16; }
-};
-
-// `bid`: number of the workgroup within its part of the launch.
-template <typename T, int DKP, bool REVERSE, bool DECAY>
-__device__ __forceinline__ void sweep_body(const SweepPair& pair, const unsigned bid) {
-    typedef Mma<T> M;
-    typedef typename M::V8 V8;
-    typedef typename M::V4 V4;
-    typedef SweepLds<DKP> L;
-    constexpr int XS = L::XS, ZS = L::ZS, NBUF = L::NBUF;
-    constexpr int KS = DKP / 32;  // 32-wide contraction steps over the feature dim
-    constexpr int KT = DKP / 16;  // 16-row state tiles
-    constexpr int XC = DKP / 64;  // 16-byte chunks per thread for an x / y tile (512 threads)
-    extern __shared__ __align__(16) unsigned char smem[];
-    T* tiles = reinterpret_cast<T*>(smem);
-    T* Ps = tiles + NBUF * L::TILE;
-    f32x4* Ob = reinterpret_cast<f32x4*>(Ps + 64 * ZS);  // [wave][i4][lane]
-
-    // Workgroups are dealt round-robin to the 8 XCDs by linear id; keep the
-    // column slices of one head on one XCD so their x / y re-reads share an L2.
-    const int xcd = bid & 7, local = bid >> 3;
-    const int nslice = pair.a[0].nslice, nprod = pair.nprod;
-    const int per_unit = nslice * pair.a[0].nchunk * nprod;
-    const int unit = xcd + 8 * (local / per_unit);
-    const int sub = local % per_unit;
-    // the sweeps of a pair alternate fastest, then the column slices, then the sequence chunks
-    const SweepArgs& a = pair.a[sub % nprod];
-    const int slice = (sub / nprod) % nslice;
-    const int chunk = sub / (nprod * nslice);
-    if (unit >= a.bh) return;
-
-    const int tid = threadIdx.x;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const bool state_role = wave >= 4;
-    const int w = wave & 3;
-    const int lane = tid & 63, r = lane & 15, g = lane >> 4;
-    const int64_t n = a.n;
-    const int dk = a.dk, dv = a.dv;
-    // one bounds-checked buffer per (batch, head) sequence; rows >= n are masked by offset below
-    const __amdgpu_buffer_rsrc_t xb = seq_rsrc<T>(a.x, a.lx, unit, a.h, n, dk);
-    const __amdgpu_buffer_rsrc_t yb = seq_rsrc<T>(a.y, a.ly, unit, a.h, n, dk);
-    const __amdgpu_buffer_rsrc_t zb = seq_rsrc<T>(a.z, a.lz, unit, a.h, n, dv);
-    const __amdgpu_buffer_rsrc_t ob = seq_rsrc<T>(a.out, a.lo, unit, a.h, n, dv);
-    const unsigned xts = (unsigned)a.lx.ts, yts = (unsigned)a.ly.ts, zts = (unsigned)a.lz.ts, ots = (unsigned)a.lo.ts;
-    const unsigned nrows = (unsigned)n;
-    const int col0 = slice * 64;  // (a.zw is 64 for this kernel)
-    const bool cols_active = (col0 + 16 * w) < dv;
-
-    float rate = 0.f;
-    if (DECAY) rate = a.s[unit % a.h];
-
-    // ---- score-wave constants: its tiles and their mask * decay factors -------
-    TileDeal deal = kDeal[w];
-    if (REVERSE) {
-        deal.itA = 3 - deal.itA; deal.jt0 = 3 - deal.jt0;
-        if (deal.itB >= 0) { deal.itB = 3 - deal.itB; deal.jt1 = 3 - deal.jt1; deal.jt2 = 3 - deal.jt2; }
-    }
-    const int itA = __builtin_amdgcn_readfirstlane(deal.itA), jt0 = __builtin_amdgcn_readfirstlane(deal.jt0);
-    const int itB = __builtin_amdgcn_readfirstlane(deal.itB), jt1 = __builtin_amdgcn_readfirstlane(deal.jt1);
-    const int jt2 = __builtin_amdgcn_readfirstlane(deal.jt2);
-    float dfac[3][4];
-    {
-        const int its[3] = {itA, itB, itB}, jts[3] = {jt0, jt1, jt2};
-#pragma unroll
-        for (int sl = 0; sl < 3; ++sl)
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int i = 16 * its[sl] + r, j = 16 * jts[sl] + 4 * g + v;
-                const int diff = REVERSE ? (j - i) : (i - j);
-                dfac[sl][v] = diff >= 0 ? (DECAY ? expf(-rate * (float)diff) : 1.f) : 0.f;
-            }
-    }
-    // ---- state-wave constants (every factor <= 1) ----------------------------
-    float ofac[4];     // scale of the inter-block term for token i = 16it + r
-    float zfac[2][8];  // scale of token j = 32ks + 8g + u in the state update
-    float lamB = 1.f;
-    if (DECAY) {
-#pragma unroll
-        for (int it = 0; it < 4; ++it) {
-            const int i = 16 * it + r;
-            ofac[it] = expf(-rate * (float)(REVERSE ? 64 - i : i));
-        }
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int j = 32 * ks + 8 * g + u;
-                zfac[ks][u] = expf(-rate * (float)(REVERSE ? j : 64 - j));
-            }
-        lamB = expf(-rate * 64.f);
-    }
-
-    f32x4 st[KT];
-    const int64_t nblk = (n + 63) / 64;
-    // Sequence chunking (chunk-parallel variant): this workgroup produces the blocks
-    // [it_first, it_end) of the walk.  Without a workspace (kWarmUp) it first runs over the blocks
-    // before it_first with the state update only ("warm-up": y and z are read, nothing is written)
-    // to rebuild the state its chunk starts from.  With one, the chunks are equally long and a
-    // workgroup walks its own chunk only: first with the state update alone, from zero, to leave the
-    // state it ends with (kCollect), then - a scan kernel having combined those into the state at the
-    // start of every chunk - for good, from that state (kApply).
-    const int mode = pair.mode;
-    const int nchunk = pair.a[0].nchunk;
-    if (mode == kCollect && chunk == nchunk - 1) return;  // nobody needs the state after the last chunk
-    const int64_t cbeg = mode == kWarmUp ? (int64_t)a.chunk_start[chunk] : min((int64_t)chunk * pair.chunk_len, nblk);
-    const int64_t cend = mode == kWarmUp ? (int64_t)a.chunk_start[chunk + 1] : min((int64_t)(chunk + 1) * pair.chunk_len, nblk);
-    const int64_t it0 = mode == kWarmUp ? 0 : cbeg;           // first block this workgroup walks
-    const int64_t it_first = mode == kCollect ? cend : cbeg;  // first block whose output it produces
-    const int64_t it_end = cend;
-    // state slots: [unit][sweep][slice][chunk 0 .. nchunk-2][state wave][tile][lane] accumulator quartets
-    constexpr size_t SF = (size_t)4 * KT * 64 * 4;
-    float* const slot0 = pair.state + ((((size_t)unit * nprod + sub % nprod) * nslice + slice) * (size_t)(nchunk - 1)) * SF;
-    const size_t lane_slot = ((size_t)w * KT * 64 + lane) * 4;
-    {
-        const bool resume = mode == kApply && chunk > 0 && state_role;
-        const float* const src = slot0 + (size_t)(chunk - 1) * SF + lane_slot;
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt)
-            st[kt] = resume ? *reinterpret_cast<const f32x4*>(src + (size_t)kt * 256) : (f32x4){0.f, 0.f, 0.f, 0.f};
-    }
-    // One register set of prefetched tiles (there are no registers to spare for two at these feature
-    // dims): while block `it` is worked on, block it+1 is in flight from memory.
-    u32x4 xrA[XC], yrA[XC], zrA;
-
-    // Per-lane byte offsets of this thread's 16-byte chunks inside a 64-token block (out of range
-    // where the chunk lies in the zero padding dk..DKP-1 or beyond dv); the block's first token goes
-    // into the wave-uniform offset of the load.  When a tile row holds a divisor of 512 chunks, a
-    // thread's chunks lie whole rows apart in the same columns and only the first one needs registers.
-    constexpr bool SAMECOL = 512 % (DKP / 8) == 0;
-    constexpr int NLANE = SAMECOL ? 1 : XC;
-    constexpr int CROWS = 512 / (DKP / 8);  // rows between two chunks of a thread (SAMECOL)
-    int lane_row[NLANE];
-    unsigned lane_x[NLANE], lane_y[NLANE];
-#pragma unroll
-    for (int u = 0; u < NLANE; ++u) {
-        const int c = tid + 512 * u;
-        const int row = c / (DKP / 8), col = (c % (DKP / 8)) * 8;
-        lane_row[u] = row;
-        lane_x[u] = col < dk ? (row * xts + col) * (unsigned)sizeof(T) : kOob;
-        lane_y[u] = col < dk ? (row * yts + col) * (unsigned)sizeof(T) : kOob;
-    }
-    const int lane_zrow = tid / 8;
-    const unsigned lane_z = (col0 + (tid % 8) * 8 < dv) ? (lane_zrow * zts + col0 + (tid % 8) * 8) * (unsigned)sizeof(T) : kOob;
-    // Fetches block number b of the walk.  Blocks at or beyond it_end, and the x tile of warm-up
-    // blocks, are fetched at the out-of-range offset: zeros, no memory traffic, and the sequence of
-    // loads is the same on every path.
-    auto load_block = [&](int64_t b, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4& zr) {
-        const int64_t t = REVERSE ? nblk - 1 - b : b;
-        const bool valid = b < it_end, need_x = valid && b >= it_first;
-        const unsigned tok0 = valid ? (unsigned)(t * 64) : 0u;
-        // rows of this block that exist (0 for a block that is not fetched)
-        const int rows = valid ? (int)min(64u, nrows - tok0) : 0, rows_x = need_x ? rows : 0;
-#pragma unroll
-        for (int u = 0; u < XC; ++u) {
-            if (SAMECOL) {
-                // a wave-uniform offset must stay inside the buffer: 0 when none of these rows exists
-                const unsigned tk = u * CROWS < rows ? tok0 + u * CROWS : 0u;
-                xr[u] = buf_load16(xb, lane_row[0] < rows_x - u * CROWS ? lane_x[0] : kOob, tk * xts * (unsigned)sizeof(T));
-                yr[u] = buf_load16(yb, lane_row[0] < rows - u * CROWS ? lane_y[0] : kOob, tk * yts * (unsigned)sizeof(T));
-            } else {
-                const int v = u < NLANE ? u : 0;
-                xr[u] = buf_load16(xb, lane_row[v] < rows_x ? lane_x[v] : kOob, tok0 * xts * (unsigned)sizeof(T));
-                yr[u] = buf_load16(yb, lane_row[v] < rows ? lane_y[v] : kOob, tok0 * yts * (unsigned)sizeof(T));
-            }
-        }
-        zr = buf_load16(zb, lane_zrow < rows ? lane_z : kOob, tok0 * zts * (unsigned)sizeof(T));
-    };
-    auto stage_block = [&](int buf, const u32x4 (&xr)[XC], const u32x4 (&yr)[XC], const u32x4& zr) {
-        T* Xd = tiles + buf * L::TILE;
-        T* Yd = Xd + 64 * XS;
-        T* Zd = Yd + 64 * XS;
-#pragma unroll
-        for (int u = 0; u < XC; ++u) {
-            const int c = tid + 512 * u;
-            const int row = c / (DKP / 8), col = (c % (DKP / 8)) * 8;
-            *reinterpret_cast<u32x4*>(Xd + row * XS + col) = xr[u];
-            *reinterpret_cast<u32x4*>(Yd + row * XS + col) = yr[u];
-        }
-        {
-            const int row = tid / 8, col = (tid % 8) * 8;
-            *reinterpret_cast<u32x4*>(Zd + row * ZS + col) = zr;
-        }
-    };
-
-    // zero P once: tiles on the masked side of the diagonal are never written
-    for (int c = tid; c < 64 * ZS / 8; c += 512) reinterpret_cast<uint4*>(Ps)[c] = make_uint4(0, 0, 0, 0);
-    load_block(it0, xrA, yrA, zrA);
-    stage_block(NBUF == 2 ? (int)(it0 & 1) : 0, xrA, yrA, zrA);
-    load_block(it0 + 1, xrA, yrA, zrA);
-    __syncthreads();
-
-    // One block of the walk.  `xr, yr, zr` hold block it+1 on entry and block it+2 on exit.
-    auto block_body = [&](const int64_t it, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4& zr) {
-        const int64_t t = REVERSE ? nblk - 1 - it : it;
-        const bool have_next = it + 1 < it_end;
-        const bool warm = it < it_first;  // warm-up block: state update only
-        const int buf = NBUF == 2 ? (int)(it & 1) : 0;
-        const T* Xs = tiles + buf * L::TILE;
-        const T* Ys = Xs + 64 * XS;
-        const T* Zs = Ys + 64 * XS;
-        // =================== phase 1 =========================================
-        if (warm) {
-            // nothing: x is not needed and no output is produced
-        } else if (!state_role) {
-            // S^T tiles of this wave -> masked, decayed P[i][j]
-            f32x4 sacc[3];
-#pragma unroll
-            for (int sl = 0; sl < 3; ++sl) sacc[sl] = (f32x4){0.f, 0.f, 0.f, 0.f};
-            const T* xa = Xs + (16 * itA + r) * XS + 8 * g;
-            const T* y0 = Ys + (16 * jt0 + r) * XS + 8 * g;
-            // all fragment reads of a batch are issued before its MFMAs (the scheduler otherwise
-            // sinks each read next to its use and the wave pays one LDS round trip per MFMA)
-            constexpr int SB = KS <= 4 ? KS : 2;  // contraction steps per batch
-            if (itB >= 0) {
-                const T* xb = Xs + (16 * itB + r) * XS + 8 * g;
-                const T* y1 = Ys + (16 * jt1 + r) * XS + 8 * g;
-                const T* y2 = Ys + (16 * jt2 + r) * XS + 8 * g;
-#pragma unroll
-                for (int k0 = 0; k0 < KS; k0 += SB) {
-                    V8 fxa[SB], fxb[SB], fy0[SB], fy1[SB], fy2[SB];
-#pragma unroll
-                    for (int ks = 0; ks < SB; ++ks) {
-                        fxa[ks] = *reinterpret_cast<const V8*>(xa + 32 * (k0 + ks));
-                        fy0[ks] = *reinterpret_cast<const V8*>(y0 + 32 * (k0 + ks));
-                        fxb[ks] = *reinterpret_cast<const V8*>(xb + 32 * (k0 + ks));
-                        fy1[ks] = *reinterpret_cast<const V8*>(y1 + 32 * (k0 + ks));
-                        fy2[ks] = *reinterpret_cast<const V8*>(y2 + 32 * (k0 + ks));
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int ks = 0; ks < SB; ++ks) {
-                        sacc[0] = M::mma(fy0[ks], fxa[ks], sacc[0]);
-                        sacc[1] = M::mma(fy1[ks], fxb[ks], sacc[1]);
-                        sacc[2] = M::mma(fy2[ks], fxb[ks], sacc[2]);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            } else {
-#pragma unroll
-                for (int k0 = 0; k0 < KS; k0 += SB) {
-                    V8 fxa[SB], fy0[SB];
-#pragma unroll
-                    for (int ks = 0; ks < SB; ++ks) {
-                        fxa[ks] = *reinterpret_cast<const V8*>(xa + 32 * (k0 + ks));
-                        fy0[ks] = *reinterpret_cast<const V8*>(y0 + 32 * (k0 + ks));
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int ks = 0; ks < SB; ++ks) sacc[0] = M::mma(fy0[ks], fxa[ks], sacc[0]);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            }
-            {
-                V4 p;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[0][v] * dfac[0][v]);
-                *reinterpret_cast<V4*>(Ps + (16 * itA + r) * ZS + 16 * jt0 + 4 * g) = p;
-            }
-            if (itB >= 0) {
-                V4 p;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[1][v] * dfac[1][v]);
-                *reinterpret_cast<V4*>(Ps + (16 * itB + r) * ZS + 16 * jt1 + 4 * g) = p;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[2][v] * dfac[2][v]);
-                *reinterpret_cast<V4*>(Ps + (16 * itB + r) * ZS + 16 * jt2 + 4 * g) = p;
-            }
-        } else if (cols_active) {
-            // inter-block term: out^T[c][i] = Lout[i] * sum_k state[k][c] x[i][k]
-            V8 sb[KS];
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    sb[ks][v] = M::cvt(st[2 * ks][v]);
-                    sb[ks][4 + v] = M::cvt(st[2 * ks + 1][v]);
-                }
-            }
-            f32x4 oacc[4];
-#pragma unroll
-            for (int i4 = 0; i4 < 4; ++i4) oacc[i4] = (f32x4){0.f, 0.f, 0.f, 0.f};
-            constexpr int IB = KS <= 4 ? KS : 2;  // contraction steps per batch of reads
-#pragma unroll
-            for (int k0 = 0; k0 < KS; k0 += IB) {
-                V8 bx[IB][4];
-#pragma unroll
-                for (int ks = 0; ks < IB; ++ks) {
-#pragma unroll
-                    for (int i4 = 0; i4 < 4; ++i4) {
-                        // two 8-byte reads from base registers the optimiser cannot relate: fused
-                        // into one ds_read2_b64 they would conflict on the LDS banks
-                        const unsigned xoff = (unsigned)((buf * L::TILE + r * XS + 32 * (k0 + ks) + 4 * g) * sizeof(T));
-                        unsigned lo = xoff, hi = xoff + 16 * (unsigned)sizeof(T);
-                        asm volatile("" : "+v"(lo));
-                        asm volatile("" : "+v"(hi));
-                        constexpr unsigned ROW = 16 * XS * (unsigned)sizeof(T);
-                        bx[ks][i4] = cat<V8, V4>(*reinterpret_cast<const V4*>(smem + lo + i4 * ROW),
-                                                 *reinterpret_cast<const V4*>(smem + hi + i4 * ROW));
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int ks = 0; ks < IB; ++ks) {
-#pragma unroll
-                    for (int i4 = 0; i4 < 4; ++i4) oacc[i4] = M::mma(sb[k0 + ks], bx[ks][i4], oacc[i4]);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-#pragma unroll
-            for (int i4 = 0; i4 < 4; ++i4) {
-                if (DECAY) {
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) oacc[i4][v] *= ofac[i4];
-                }
-                Ob[(w * 4 + i4) * 64 + lane] = oacc[i4];
-            }
-        }
-        if (!warm) __syncthreads();  // warm-up blocks share nothing between the two phases
-
-        // =================== phase 2 =========================================
-        if (!state_role) {
-            if (cols_active && !warm) {
-                // out^T = inter + z^T P^T, then store out[token][16w + 4g .. +3]
-                V8 zf[2];
-#pragma unroll
-                for (int ks = 0; ks < 2; ++ks) {
-                    const T* pz = Zs + (32 * ks + 8 * g + (r >> 2)) * ZS + 16 * w + 4 * (r & 3);
-                    zf[ks] = cat<V8, V4>(lds_tr4<V4>(pz), lds_tr4<V4>(pz + 4 * ZS));
-                }
-                f32x4 oacc[4];
-#pragma unroll
-                for (int i4 = 0; i4 < 4; ++i4) oacc[i4] = Ob[(w * 4 + i4) * 64 + lane];
-                V8 bp[4][2];
-#pragma unroll
-                for (int i4 = 0; i4 < 4; ++i4) {
-#pragma unroll
-                    for (int ks = 0; ks < 2; ++ks) {
-                        const bool need = REVERSE ? (ks >= i4 / 2) : (ks <= i4 / 2);
-                        if (need) bp[i4][ks] = *reinterpret_cast<const V8*>(Ps + (16 * i4 + r) * ZS + 32 * ks + 8 * g);
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int i4 = 0; i4 < 4; ++i4) {
-#pragma unroll
-                    for (int ks = 0; ks < 2; ++ks) {
-                        const bool need = REVERSE ? (ks >= i4 / 2) : (ks <= i4 / 2);
-                        if (need) oacc[i4] = M::mma(zf[ks], bp[i4][ks], oacc[i4]);
-                    }
-                }
-                const int col = col0 + 16 * w + 4 * g;
-#pragma unroll
-                for (int i4 = 0; i4 < 4; ++i4) {
-                    const unsigned tok = (unsigned)(t * 64) + 16 * i4;  // wave-uniform first token of the tile
-                    V4 o;
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) o[v] = (T)oacc[i4][v];
-                    const unsigned off = (col < dv && tok + r < nrows) ? (r * ots + col) * (unsigned)sizeof(T) : kOob;
-                    buf_store8(ob, off, tok < nrows ? tok * ots * (unsigned)sizeof(T) : 0u, __builtin_bit_cast(u32x2, o));
-                }
-            }
-        } else if (cols_active && (have_next || mode == kCollect)) {
-            // state = lam^64 state + y^T (z * Lupd)
-            V8 zf[2];
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                const T* pz = Zs + (32 * ks + 8 * g + (r >> 2)) * ZS + 16 * w + 4 * (r & 3);
-                zf[ks] = cat<V8, V4>(lds_tr4<V4>(pz), lds_tr4<V4>(pz + 4 * ZS));
-            }
-            constexpr int UB = KT <= 8 ? KT : 4;  // state tiles per batch of transposed reads
-#pragma unroll
-            for (int t0 = 0; t0 < KT; t0 += UB) {
-                V8 ay[UB][2];
-#pragma unroll
-                for (int kt = 0; kt < UB; ++kt) {
-#pragma unroll
-                    for (int ks = 0; ks < 2; ++ks) {
-                        const T* py = Ys + (32 * ks + 8 * g + (r >> 2)) * XS + 16 * (t0 + kt) + 4 * (r & 3);
-                        ay[kt][ks] = cat<V8, V4>(lds_tr4<V4>(py), lds_tr4<V4>(py + 4 * XS));
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-                if (DECAY && t0 == 0) {
-#pragma unroll
-                    for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) zf[ks][u] = (T)((float)zf[ks][u] * zfac[ks][u]);
-#pragma unroll
-                    for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-                        for (int v = 0; v < 4; ++v) st[kt][v] *= lamB;
-                }
-#pragma unroll
-                for (int kt = 0; kt < UB; ++kt) {
-#pragma unroll
-                    for (int ks = 0; ks < 2; ++ks) st[t0 + kt] = M::mma(ay[kt][ks], zf[ks], st[t0 + kt]);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-        if (NBUF == 2) {
-            stage_block((int)((it + 1) & 1), xr, yr, zr);
-            load_block(it + 2, xr, yr, zr);
-            __syncthreads();
-        } else {
-            __syncthreads();
-            stage_block(0, xr, yr, zr);
-            load_block(it + 2, xr, yr, zr);
-            __syncthreads();
-        }
-    };
-    for (int64_t it = it0; it < it_end; ++it) block_body(it, xrA, yrA, zrA);
-    if (mode == kCollect && state_role) {
-        float* const dst = slot0 + (size_t)chunk * SF + lane_slot;
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<f32x4*>(dst + (size_t)kt * 256) = st[kt];
-    }
-}
-
-template <typename T, int DKP, bool REVERSE, bool DECAY>
-__global__ __launch_bounds__(512, 1) void la_sweep_kernel(SweepPair pair) {
-    sweep_body<T, DKP, REVERSE, DECAY>(pair, blockIdx.x);
-}
-
-// Forward-walking and backward-walking sweeps in one launch (SweepBoth).
-template <typename T, int DKP, bool DECAY>
-__global__ __launch_bounds__(512, 1) void la_sweep_both_kernel(SweepBoth both) {
-    if (blockIdx.x < both.nfwd) sweep_body<T, DKP, false, DECAY>(both.fwd, blockIdx.x);
-    else sweep_body<T, DKP, true, DECAY>(both.rev, blockIdx.x - both.nfwd);
-}
-
-static unsigned part_grid(const SweepPair& p) {
-    return (unsigned)((p.a[0].bh + 7) / 8 * 8 * p.a[0].nslice * p.a[0].nchunk * p.nprod);
-}
-
-template <typename T, int DKP, bool DECAY>
-static int launch_both_one(const SweepBoth& b, hipStream_t st) {
-    constexpr size_t lds = SweepLds<DKP>::bytes(sizeof(T));
-    auto kern = la_sweep_both_kernel<T, DKP, DECAY>;
-    static unsigned char lds_allowed[kMaxDevices];
-    if (const int e = allow_lds(kern, lds, lds_allowed)) return e;
-    hipLaunchKernelGGL(kern, dim3(b.nfwd + part_grid(b.rev)), dim3(512), lds, st, b);
-    return (int)hipGetLastError();
-}
-
-template <typename T>
-static int launch_both(const SweepBoth& b, hipStream_t st) {
-    const bool decay = b.fwd.a[0].s != nullptr;
-#define LA_GO(DKP) (decay ? launch_both_one<T, DKP, true>(b, st) : launch_both_one<T, DKP, false>(b, st))
-    if (b.fwd.a[0].dk <= 192) return LA_GO(192);
-    return LA_GO(256);
-#undef LA_GO
-}
-
-template <typename T, int DKP, bool REVERSE, bool DECAY>
-static int launch_one(const SweepPair& pair, hipStream_t st) {
-    const SweepArgs& a = pair.a[0];
-    if (pair.mode != kWarmUp && pipe_state_floats(a.dk, false) != (size_t)4 * (DKP / 16) * 64 * 4) return LA_E_WORKSPACE;
-    constexpr size_t lds = SweepLds<DKP>::bytes(sizeof(T));
-    static_assert(lds <= 160 * 1024, "LDS budget");
-    auto kern = la_sweep_kernel<T, DKP, REVERSE, DECAY>;
-    static unsigned char lds_allowed[kMaxDevices];
-    if (const int e = allow_lds(kern, lds, lds_allowed)) return e;
-    const int units8 = (a.bh + 7) / 8 * 8;
-    const unsigned grid = (unsigned)(units8 * a.nslice * a.nchunk * pair.nprod);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, st, pair);
-    return (int)hipGetLastError();
-}
-
-template <typename T, bool REVERSE>
-static int launch_dir(const SweepPair& pair, hipStream_t st) {
-    const SweepArgs& a = pair.a[0];
-    const bool decay = a.s != nullptr;
-#define LA_GO(DKP) (decay ? launch_one<T, DKP, REVERSE, true>(pair, st) : launch_one<T, DKP, REVERSE, false>(pair, st))
-    if (a.dk <= 192) return LA_GO(192);
-    return LA_GO(256);
-#undef LA_GO
-}
-
+// Compute units of the current device, asked once per device.
 static int num_cus() {
-    static const int cus = [] {
-        int dev = 0, n = 256;
-        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
-        return n > 0 ? n : 256;
-    }();
-    return cus;
+    static int cache[kMaxDevices];  // 0: not asked yet
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    const bool cached = dev >= 0 && dev < kMaxDevices;
+    if (cached) {
+        const int c = __atomic_load_n(&cache[dev], __ATOMIC_RELAXED);
+        if (c > 0) return c;
+    }
+    int n = 256;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    if (cached) __atomic_store_n(&cache[dev], n, __ATOMIC_RELAXED);
+    return n;
 }
 
 // Sequence chunks per (batch, head, slice).  With few sequences a single sweep per sequence
@@ -582,29 +86,6 @@ static SweepArgs make_args(const SweepIO& io, const float* s, int64_t bh, int64_
     return a;
 }
 
-static int launch_classic_one(const SweepPair& p, int dtype, bool reverse, hipStream_t st) {
-    if (dtype == LA_BF16) return reverse ? launch_dir<__bf16, true>(p, st) : launch_dir<__bf16, false>(p, st);
-    if (dtype == LA_FP16) return reverse ? launch_dir<_Float16, true>(p, st) : launch_dir<_Float16, false>(p, st);
-    return LA_E_UNSUPPORTED;
-}
-
-// The two-barrier kernel (feature dims 129..256), in one launch or - chunks with scanned states - three.
-static int launch_classic(const SweepPair& p, int dtype, bool reverse, hipStream_t st) {
-    SweepPair q = p;
-    if (p.mode == kWarmUp || p.a[0].nchunk <= 1) {
-        q.mode = kWarmUp;
-        return launch_classic_one(q, dtype, reverse, st);
-    }
-    if (!p.state || p.chunk_len < 1) return LA_E_WORKSPACE;
-    q.mode = kCollect;
-    int rc = launch_classic_one(q, dtype, reverse, st);
-    if (rc != LA_OK) return rc;
-    rc = launch_state_scan(p, st);
-    if (rc != LA_OK) return rc;
-    q.mode = kApply;
-    return launch_classic_one(q, dtype, reverse, st);
-}
-
 // With a workspace the kernels do not rebuild a chunk's incoming state with warm-up blocks: the states
 // the chunks end with are collected and scanned, and every chunk starts from the result (three
 // launches; equally long chunks, up to 64 of them).  Number of chunks and bytes of workspace for a
@@ -626,12 +107,9 @@ static double block_us(int64_t dk, bool wide) {
     if (dk <= 192) return wide ? 3.0 : 2.1;
     return wide ? 4.1 : 2.9;
 }
-// Column slices per sequence: 64 columns each, or - wide - 128 (feature dim up to 128), 96 (up to 192), 128 (up to 256).
-static int64_t wide_slices(int64_t dk, int64_t dv) {
-    const int64_t zw = dk <= 128 ? 128 : wide_zw_max((int)dk);
-    return (dv + zw - 1) / zw;
-}
-static int64_t slices(int64_t dk, int64_t dv, bool wide) { return wide ? wide_slices(dk, dv) : (dv + 63) / 64; }
+// Column slices per sequence: 64 columns each, or - wide - 128.
+static int64_t wide_slices(int64_t dv) { return (dv + 127) / 128; }
+static int64_t slices(int64_t dk, int64_t dv, bool wide) { return wide ? wide_slices(dv) : (dv + 63) / 64; }
 static double warm_up_frac(int64_t wgs, int64_t nblk) {
     static const double frac[9] = {1.0, 1.0, 0.77, 0.71, 0.68, 0.67, 0.66, 0.66, 0.66};
     return frac[warm_up_chunks(wgs, nblk)];
@@ -675,11 +153,11 @@ static ScanPlan plan_scan(int64_t bh, int64_t n, int64_t dk, int64_t dv, int npr
 // `scratch`: bytes of workspace the caller has.  opts.wide overrides the choice.
 static bool wide_columns(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, size_t scratch, const Opts& opts) {
     if (dk > 128) {
-        // Two-barrier kernels: 96- / 128-column workgroups (la_sweep_wide.hip) where that makes fewer slices.
+        // Feature dims 129 .. 256: 128-column workgroups where that makes fewer slices.
         // They pay when the 64-column form needs more rounds of workgroups than the chip has CUs for
         // (a wide workgroup takes about 1.4 times as long); with few sequences the 64-column form has
         // more workgroups to spread over the CUs and stays.
-        const int64_t ws = wide_slices(dk, dv), ns = (dv + 63) / 64;
+        const int64_t ws = wide_slices(dv), ns = (dv + 63) / 64;
         if (ws >= ns) return false;
         if (opts.wide != LA_OPT_AUTO) return opts.wide == LA_OPT_ON;
         const int64_t cus = num_cus(), units = (bh + 7) / 8 * 8 * nprod, wide = units * ws, narrow = units * ns;
@@ -716,10 +194,10 @@ static int launch_planned(SweepPair& p, int64_t bh, int64_t n, int64_t dk, int64
     p.state = nullptr;
     for (int i = 0; i < p.nprod; ++i)
         if (p.wide) {
-            const int64_t ws = wide_slices(dk, dv);
+            // equal slices, a whole number of 32-column state waves each (192 columns: 96 + 96, not 128 + 64)
+            const int64_t ws = wide_slices(dv);
             p.a[i].nslice = (int)ws;
-            // equal slices, a whole number of 32-column state waves each
-            p.a[i].zw = dk <= 128 ? 128 : (int)(((dv + ws - 1) / ws + 31) / 32 * 32);
+            p.a[i].zw = (int)(((dv + ws - 1) / ws + 31) / 32 * 32);
         }
     const ScanPlan pl = plan_scan(bh, n, dk, dv, p.nprod, p.wide != 0, opts);
     if (pl.nchunk > 1 && ws_ok && ws_bytes >= pl.bytes) {
@@ -738,9 +216,7 @@ static int launch_planned(SweepPair& p, int64_t bh, int64_t n, int64_t dk, int64
         }
     }
     if (p.nprod == 1) p.a[1] = p.a[0];
-    if (dk <= 128) return sweep_pipe(p, dtype, reverse, st);  // pipelined kernel, la_sweep_pipe.hip
-    if (p.wide) return sweep_wide(p, dtype, reverse, st);     // 96- / 128-column workgroups, la_sweep_wide.hip
-    return launch_classic(p, dtype, reverse, st);
+    return sweep_pipe(p, dtype, reverse, st);
 }
 
 // x,y: (b,h,n,dk)  z,out: (b,h,n,dv), each with its own batch / head / token strides
@@ -887,9 +363,7 @@ int sweep_bwd_once(const SweepIO& dq, const SweepIO& dk, const SweepIO& dv, cons
         for (int j = 0; j < 9; ++j) b.rev.a[i].chunk_start[j] = b.fwd.a[0].chunk_start[j];
     }
     b.nfwd = part_grid(b.fwd);
-    if (d <= 128) return sweep_pipe_both(b, dtype, st);
-    if (dtype == LA_BF16) return launch_both<__bf16>(b, st);
-    return launch_both<_Float16>(b, st);
+    return sweep_pipe_both(b, dtype, st);
 }
 
 // The same for two sweeps of one shape and opposite directions (dQ and dK of a backward pass with
@@ -926,9 +400,7 @@ int sweep_fwd_rev_once(const SweepIO& fwd, const SweepIO& rev, const float* s, i
         p->state = nullptr;
     }
     b.nfwd = part_grid(b.fwd);
-    if (dk <= 128) return sweep_pipe_both(b, dtype, st);
-    if (dtype == LA_BF16) return launch_both<__bf16>(b, st);
-    return launch_both<_Float16>(b, st);
+    return sweep_pipe_both(b, dtype, st);
 }
 
 }  // namespace la

@@ -24,7 +24,7 @@ struct SweepArgs {
     const float* s; // h decay rates or nullptr
     int64_t n;
     int dk, dv, h, bh, nslice;
-    int zw;              // columns of z / out per slice (la_sweep.hip: 64; la_sweep_wide.hip: a multiple of 32 up to 128)
+    int zw;              // columns of z / out per slice: 64, or - 128-column workgroups - a multiple of 32 up to 128
     int nchunk;          // sequence chunks per (batch, head, slice); 1 = one workgroup walks the whole sequence
     int chunk_start[9];  // first 64-token block (in walk order) of each chunk; chunk_start[nchunk] = number of blocks
 };
@@ -136,7 +136,11 @@ struct SweepBoth {
     SweepPair fwd, rev;
     unsigned nfwd;  // workgroups of the forward part (a multiple of 8); the reverse part follows
 };
-int sweep_pipe_both(const SweepBoth& b, int dtype, hipStream_t st);  // feature dim up to 128, la_sweep_pipe.hip
+int sweep_pipe_both(const SweepBoth& b, int dtype, hipStream_t st);  // la_sweep_pipe.hip
+// Workgroups of one part of such a launch (units are dealt to the 8 XCDs, so their number is rounded up to 8).
+inline unsigned part_grid(const SweepPair& p) {
+    return (unsigned)((p.a[0].bh + 7) / 8 * 8 * p.a[0].nslice * p.a[0].nchunk * p.nprod);
+}
 
 // Count (up to 8) and first blocks, chunk_start[0 .. 8], of the warm-up chunks for a launch that would have
 // `wgs` workgroups with one chunk each, on a walk of nblk blocks; `forced` > 0 overrides the count.
@@ -167,22 +171,17 @@ struct SavedPlan {
     size_t bytes;
 };
 
-// Launches the single-barrier pipelined kernel (feature dim up to 128); defined in la_sweep_pipe.hip.
+// Launches the single-barrier pipelined kernel (feature dim up to 256); defined in la_sweep_pipe.hip.
 // n, dk, dv, h, bh, nslice and the chunking must agree between the two sweeps of a pair.
 enum { kWarmUp = 0, kCollect = 1, kApply = 2, kResume = 3 };
 int sweep_pipe(const SweepPair& p, int dtype, bool reverse, hipStream_t st);
-// Floats of one state slot: the feature dim as the kernel pads it (64 or 128 in the pipelined kernel, 192
-// or 256 in the two-barrier one) times the 64 or 128 columns of a workgroup.  Must agree with the
-// kernels' own SF; the 128-column form exists for the 128-wide feature tile only.
+// Floats of one state slot: the feature dim as the kernel pads it (64, 128, 192 or 256) times the 64 or 128
+// columns of a workgroup.  Must agree with the kernels' own SF; the 128-column form pads feature dims up
+// to 64 to 128.
 inline size_t pipe_state_floats(int dk, bool wide) {
     const int dkp = dk > 192 ? 256 : dk > 128 ? 192 : (dk <= 64 && !wide ? 64 : 128);
     return (size_t)dkp * (wide ? 128 : 64);
 }
 // Between a kCollect and a kApply launch: scans the chunks' end states in place (la_sweep_pipe.hip).
 int launch_state_scan(const SweepPair& p, hipStream_t st);
-// Launches the two-barrier kernel with 96- / 128-column workgroups (feature dims 129 .. 256); la_sweep_wide.hip.
-int sweep_wide(const SweepPair& p, int dtype, bool reverse, hipStream_t st);
-// Columns per workgroup that kernel can take at a feature dim.
-inline int wide_zw_max(int dk) { return dk <= 192 ? 96 : 128; }
-
 }  // namespace la

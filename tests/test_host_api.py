@@ -227,3 +227,26 @@ def test_triton_import_path_is_an_alias_of_the_hip_operators():
     for f in (a1, a2, a3, b1, b2, b3):
         assert callable(f)
     assert a1.__self__ is hip.LightningAttention2 and a2.__self__ is hip.LightningAttention2NoDecay
+
+
+def test_triton_package_names_stay_operators_after_submodule_imports():
+    """Importing a submodule first (as `from lightning_attn.ops.triton.lightning_attn2 import ...` does) must not
+    turn the package attribute of the same name into the module: checked in a fresh interpreter."""
+    import subprocess
+    import sys
+
+    code = (
+        "import sys; sys.path[:0] = %r\n"
+        "import lightning_attn.ops.triton.lightning_attn2\n"
+        "import lightning_attn.ops.triton.lightning_attn2_no_decay\n"
+        "import lightning_attn.ops.triton.lightning_attn2_parallel\n"
+        "import lightning_attn.ops.triton.srmsnorm\n"
+        "import lightning_attn.ops.triton as t\n"
+        "from lightning_attn.ops.triton import lightning_attn2, lightning_attn2_no_decay, lightning_attn2_parallel\n"
+        "import types\n"
+        "for f in (lightning_attn2, lightning_attn2_no_decay, lightning_attn2_parallel, t.lightning_attn2):\n"
+        "    assert callable(f) and not isinstance(f, types.ModuleType), f\n"
+        "assert isinstance(t.SimpleRMSNorm, type)\n"
+    ) % (sys.path[:2],)
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
