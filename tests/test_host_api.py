@@ -232,9 +232,11 @@ def test_triton_import_path_is_an_alias_of_the_hip_operators():
 def test_triton_package_names_stay_operators_after_submodule_imports():
     """Importing a submodule first (as `from lightning_attn.ops.triton.lightning_attn2 import ...` does) must not
     turn the package attribute of the same name into the module: checked in a fresh interpreter."""
+    import os
     import subprocess
     import sys
 
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     code = (
         "import sys; sys.path[:0] = %r\n"
         "import lightning_attn.ops.triton.lightning_attn2\n"
@@ -247,6 +249,6 @@ def test_triton_package_names_stay_operators_after_submodule_imports():
         "for f in (lightning_attn2, lightning_attn2_no_decay, lightning_attn2_parallel, t.lightning_attn2):\n"
         "    assert callable(f) and not isinstance(f, types.ModuleType), f\n"
         "assert isinstance(t.SimpleRMSNorm, type)\n"
-    ) % (sys.path[:2],)
+    ) % ([os.path.join(root, "lightning-attention_amd"), root],)
     r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr
