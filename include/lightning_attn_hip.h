@@ -18,9 +18,17 @@
  *   - dtype: LA_BF16 = 0, LA_FP16 = 1, LA_FP32 = 2 (element type of q,k,v,o and
  *     of the gradients; x,y,dy,dx for the norm).  Slopes, rstd and every
  *     accumulator are float32;
- *   - calls are re-entrant and thread-safe: the library keeps no mutable state and reads
- *     nothing from the process environment; how a call is mapped onto launches depends on
- *     its arguments alone (la_launch_opts below, where a caller wants to override that).
+ *   - nothing is read from the process environment: how a call is mapped onto launches depends on
+ *     its arguments (la_launch_opts below, where a caller wants to override the library's choices)
+ *     and on the compute-unit count of the current device;
+ *   - calls are thread-safe and may overlap on different streams, with one exception: la_fwd_static,
+ *     whose calls share one scratch array per GPU (one call in flight per GPU, see there);
+ *   - what the library remembers, per device and until the process ends: the device's compute-unit
+ *     count (asked once; launch plans and workspace sizes depend on it), one flag per kernel
+ *     instantiation saying that its dynamic-LDS limit has been raised (hipFuncSetAttribute, made before
+ *     that kernel's first launch) and the address of la_fwd_static's array.  The first use of a kernel on a
+ *     device therefore does more than enqueue work, which stream capture does not allow: call la_init()
+ *     on the device beforehand, or make the first call of each shape outside the capture.
  */
 #ifndef LIGHTNING_ATTN_HIP_H
 #define LIGHTNING_ATTN_HIP_H
@@ -42,6 +50,16 @@ enum {
     LA_E_WORKSPACE = -4,   /* workspace too small for the requested plan       */
     LA_E_ALIGN = -5        /* a pointer or stride is not 16-byte aligned      */
 };
+
+/*
+ * One-time work for the current device, done up front instead of at first use: the compute-unit count,
+ * the dynamic-LDS limit of every kernel instantiation and the address of la_fwd_static's array.  After it
+ * every other entry point only enqueues kernels on that device, so first calls may sit inside a stream
+ * capture.  Optional otherwise; idempotent; returns 0 or the hipError_t of the failing runtime call.
+ * No counterpart in the reference (Triton compiles and configures its kernels at their first launch,
+ * lightning_attn/ops/triton/lightning_attn2.py:416).
+ */
+int la_init(void);
 
 /* Host-only helpers (usable without a GPU). */
 const char *la_version(void);

@@ -19,6 +19,8 @@ int sweep_saving(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64
                  float* save, int save_len, hipStream_t st);
 int sweep_resumed(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
                   const float* saved, int nchunk, int chunk_len, hipStream_t st);
+int prepare_srmsnorm();   // srmsnorm.hip
+int prepare_norm_gate();  // norm_gate.hip
 int sweep_f32(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
               int64_t n, int64_t dk, int64_t dv, bool reverse, int chunks, hipStream_t st);
 int sweep_f32_bwd_once(const void* q, const void* k, const void* v, const void* dout, void* dq, void* dk, void* dv,
@@ -308,6 +310,17 @@ static int static_scratch(void** out) {
     return LA_OK;
 }
 }  // namespace la
+
+extern "C" int la_init(void) {
+    int rc = la::prepare_plans();
+    if (rc == LA_OK) rc = la::prepare_pipe();
+    if (rc == LA_OK) rc = la::prepare_f32();
+    if (rc == LA_OK) rc = la::prepare_srmsnorm();
+    if (rc == LA_OK) rc = la::prepare_norm_gate();
+    void* p = nullptr;
+    if (rc == LA_OK) rc = la::static_scratch(&p);
+    return rc;
+}
 
 extern "C" int la_fwd_static(const void* q, const void* k, const void* v, const float* s, void* o, int64_t b, int64_t h,
                              int64_t n, int64_t d, int64_t e, int dtype, void* stream) {

@@ -59,6 +59,24 @@ struct ElemTraits<float> {
     static constexpr int kDtype = 2;
 };
 
+// Compute units of the current device (256 if it cannot be asked), asked once per device: launch plans and
+// workspace sizes depend on it.
+constexpr int kMaxDevices = 64;
+inline int num_cus() {
+    static int cache[kMaxDevices];  // 0: not asked yet
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    const bool cached = dev >= 0 && dev < kMaxDevices;
+    if (cached) {
+        const int c = __atomic_load_n(&cache[dev], __ATOMIC_RELAXED);
+        if (c > 0) return c;
+    }
+    int n = 256;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    if (cached) __atomic_store_n(&cache[dev], n, __ATOMIC_RELAXED);
+    return n;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);

@@ -17,21 +17,7 @@
 
 namespace la {
 
-// Compute units of the current device, asked once per device.
-static int num_cus() {
-    static int cache[kMaxDevices];  // 0: not asked yet
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return 256;
-    const bool cached = dev >= 0 && dev < kMaxDevices;
-    if (cached) {
-        const int c = __atomic_load_n(&cache[dev], __ATOMIC_RELAXED);
-        if (c > 0) return c;
-    }
-    int n = 256;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    if (cached) __atomic_store_n(&cache[dev], n, __ATOMIC_RELAXED);
-    return n;
-}
+int prepare_plans() { return num_cus() > 0 ? 0 : (int)hipErrorInvalidDevice; }
 
 // Sequence chunks per (batch, head, slice).  With few sequences a single sweep per sequence
 // leaves most of the 256 CUs idle; the walk is then cut into up to 8 chunks whose workgroups

@@ -149,7 +149,6 @@ void plan_warm_up_chunks(int64_t wgs, int64_t nblk, int forced, int* nchunk, int
 
 // Raises a kernel's dynamic LDS limit above the 64 KB default, once per kernel and device (the call is
 // not free and the limit stays).  `done` is the instantiation's own flag array, one entry per device.
-constexpr int kMaxDevices = 64;
 template <typename K>
 inline int allow_lds(K kern, size_t lds, unsigned char (&done)[kMaxDevices]) {
     if (lds <= 64 * 1024) return 0;
@@ -175,6 +174,12 @@ struct SavedPlan {
 // n, dk, dv, h, bh, nslice and the chunking must agree between the two sweeps of a pair.
 enum { kWarmUp = 0, kCollect = 1, kApply = 2, kResume = 3 };
 int sweep_pipe(const SweepPair& p, int dtype, bool reverse, hipStream_t st);
+// One-time work per device, done ahead of the first launches: the dynamic LDS limits of every instantiation
+// of the pipelined kernels (la_sweep_pipe.hip) and of the float32 kernels (la_sweep_f32.hip), and the
+// device's compute-unit count (la_sweep.hip).
+int prepare_pipe();
+int prepare_f32();
+int prepare_plans();
 // Floats of one state slot: the feature dim as the kernel pads it (64, 128, 192 or 256) times the 64 or 128
 // columns of a workgroup.  Must agree with the kernels' own SF; the 128-column form pads feature dims up
 // to 64 to 128.

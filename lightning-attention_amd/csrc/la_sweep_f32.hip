@@ -279,11 +279,34 @@ __global__ __launch_bounds__(256, DKP <= 64 ? 2 : 1) void la_sweep_f32_trio_kern
 }
 
 template <int DKP, bool DECAY>
+static int prep_trio_f32() {
+    constexpr size_t lds = (size_t)(2 * 64 * (DKP + LA_F32_XPAD) + 2 * 64 * 68) * sizeof(float);
+    static unsigned char lds_allowed[kMaxDevices];
+    return allow_lds(la_sweep_f32_trio_kernel<DKP, DECAY>, lds, lds_allowed);
+}
+template <int DKP, bool REVERSE, bool DECAY>
+static int prep_one_f32() {
+    constexpr size_t lds = (size_t)(2 * 64 * (DKP + LA_F32_XPAD) + 2 * 64 * 68) * sizeof(float);
+    static unsigned char lds_allowed[kMaxDevices];
+    return allow_lds(la_sweep_f32_kernel<DKP, REVERSE, DECAY>, lds, lds_allowed);
+}
+// Every instantiation of this file made ready for its first launch on the current device.
+int prepare_f32() {
+    int e = 0;
+#define LA_P(DKP, D) \
+    if (!e) e = prep_trio_f32<DKP, D>(); \
+    if (!e) e = prep_one_f32<DKP, false, D>(); \
+    if (!e) e = prep_one_f32<DKP, true, D>();
+    LA_P(64, false) LA_P(64, true) LA_P(128, false) LA_P(128, true)
+#undef LA_P
+    return e;
+}
+
+template <int DKP, bool DECAY>
 static int launch_trio_f32(const SweepTrioF32& t, hipStream_t st) {
     constexpr size_t lds = (size_t)(2 * 64 * (DKP + LA_F32_XPAD) + 2 * 64 * 68) * sizeof(float);
     auto kern = la_sweep_f32_trio_kernel<DKP, DECAY>;
-    static unsigned char lds_allowed[kMaxDevices];
-    if (const int e = allow_lds(kern, lds, lds_allowed)) return e;
+    if (const int e = prep_trio_f32<DKP, DECAY>()) return e;
     hipLaunchKernelGGL(kern, dim3(3 * t.per_part), dim3(256), lds, st, t);
     return (int)hipGetLastError();
 }
@@ -292,8 +315,7 @@ template <int DKP, bool REVERSE, bool DECAY>
 static int launch_one_f32(const SweepArgsF32& a, hipStream_t st) {
     constexpr size_t lds = (size_t)(2 * 64 * (DKP + LA_F32_XPAD) + 2 * 64 * 68) * sizeof(float);
     auto kern = la_sweep_f32_kernel<DKP, REVERSE, DECAY>;
-    static unsigned char lds_allowed[kMaxDevices];
-    if (const int e = allow_lds(kern, lds, lds_allowed)) return e;
+    if (const int e = prep_one_f32<DKP, REVERSE, DECAY>()) return e;
     const int units8 = (a.bh + 7) / 8 * 8;
     hipLaunchKernelGGL(kern, dim3((unsigned)(units8 * a.nslice * a.nchunk)), dim3(256), lds, st, a);
     return (int)hipGetLastError();

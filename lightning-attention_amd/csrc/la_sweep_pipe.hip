@@ -89,6 +89,18 @@ static int launch_any(const SweepPair& p, int dtype, bool reverse, hipStream_t s
     return LA_E_UNSUPPORTED;
 }
 
+// Every instantiation of the pipelined kernel made ready for its first launch on the current device.
+int prepare_pipe() {
+    int e = prep_family<__bf16, 64, 1, 1>();
+    if (!e) e = prep_family<__bf16, 128, 1, 1>();
+    if (!e) e = prep_family<__bf16, 128, 1, 2>();
+    if (!e) e = prep_family<_Float16, 64, 1, 1>();
+    if (!e) e = prep_family<_Float16, 128, 1, 1>();
+    if (!e) e = prep_family<_Float16, 128, 1, 2>();
+    if (!e) e = prepare_split();
+    return e;
+}
+
 int sweep_pipe(const SweepPair& p, int dtype, bool reverse, hipStream_t st) {
     const SweepArgs& a = p.a[0];
     if (a.dk > 256 || p.nprod < 1 || p.nprod > 2) return LA_E_UNSUPPORTED;

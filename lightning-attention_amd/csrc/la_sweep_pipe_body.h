@@ -740,14 +740,21 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_both_kernel(SweepBoth bo
     else sweep_pipe_body<T, DKP, NF, 1, true, DECAY, DENSE>(both.rev, blockIdx.x - both.nfwd);
 }
 
+// What a kernel instantiation needs once per device before its first launch (its dynamic LDS limit raised).
+template <typename T, int DKP, int NF, int NH, bool REVERSE, bool DECAY, bool DENSE>
+static int prep_one() {
+    constexpr size_t lds = PipeLds<DKP, NF, NH>::bytes(sizeof(T));
+    static_assert(lds <= 160 * 1024, "LDS budget");
+    static unsigned char lds_allowed[kMaxDevices];
+    return allow_lds(la_sweep_pipe_kernel<T, DKP, NF, NH, REVERSE, DECAY, DENSE>, lds, lds_allowed);
+}
+
 template <typename T, int DKP, int NF, int NH, bool REVERSE, bool DECAY, bool DENSE>
 static int launch_one(const SweepPair& pair, hipStream_t st) {
     const SweepArgs& a = pair.a[0];
     constexpr size_t lds = PipeLds<DKP, NF, NH>::bytes(sizeof(T));
-    static_assert(lds <= 160 * 1024, "LDS budget");
     auto kern = la_sweep_pipe_kernel<T, DKP, NF, NH, REVERSE, DECAY, DENSE>;
-    static unsigned char lds_allowed[kMaxDevices];
-    if (const int e = allow_lds(kern, lds, lds_allowed)) return e;
+    if (const int e = prep_one<T, DKP, NF, NH, REVERSE, DECAY, DENSE>()) return e;
     const int units8 = (a.bh + 7) / 8 * 8;
     // the slice width the host chose must be one this instantiation's LDS slot and state waves hold
     if (a.zw <= 0 || a.zw > 64 * NH || a.zw % (16 * NH)) return LA_E_UNSUPPORTED;
@@ -776,17 +783,40 @@ static inline bool all_plain(const SweepPair& p) {
 }
 
 template <typename T, int DKP, int NF, bool DECAY, bool DENSE>
+static int prep_both_one() {
+    constexpr size_t lds = PipeLds<DKP, NF, 1>::bytes(sizeof(T));
+    static unsigned char lds_allowed[kMaxDevices];
+    return allow_lds(la_sweep_pipe_both_kernel<T, DKP, NF, DECAY, DENSE>, lds, lds_allowed);
+}
+
+template <typename T, int DKP, int NF, bool DECAY, bool DENSE>
 static int launch_both_one(const SweepBoth& b, hipStream_t st) {
     constexpr size_t lds = PipeLds<DKP, NF, 1>::bytes(sizeof(T));
     auto kern = la_sweep_pipe_both_kernel<T, DKP, NF, DECAY, DENSE>;
-    static unsigned char lds_allowed[kMaxDevices];
-    if (const int e = allow_lds(kern, lds, lds_allowed)) return e;
+    if (const int e = prep_both_one<T, DKP, NF, DECAY, DENSE>()) return e;
     hipLaunchKernelGGL(kern, dim3(b.nfwd + part_grid(b.rev)), dim3(512), lds, st, b);
     return (int)hipGetLastError();
+}
+
+// prep_one / prep_both_one for every direction, decay and layout form of one (element type, shape) family.
+template <typename T, int DKP, int NF, int NH>
+static int prep_family() {
+    int e = 0;
+#define LA_P(R, D, S) if (!e) e = prep_one<T, DKP, NF, NH, R, D, S>();
+    LA_P(false, false, false) LA_P(false, false, true) LA_P(false, true, false) LA_P(false, true, true)
+    LA_P(true, false, false) LA_P(true, false, true) LA_P(true, true, false) LA_P(true, true, true)
+#undef LA_P
+    if (NH == 1) {
+#define LA_P(D, S) if (!e) e = prep_both_one<T, DKP, NF, D, S>();
+        LA_P(false, false) LA_P(false, true) LA_P(true, false) LA_P(true, true)
+#undef LA_P
+    }
+    return e;
 }
 
 // The instantiations for feature dims 129 .. 256 live in a translation unit of their own (la_sweep_pipe_split.hip).
 int launch_split(const SweepPair& p, int dtype, bool reverse, hipStream_t st);
 int launch_split_both(const SweepBoth& b, int dtype, hipStream_t st);
+int prepare_split();
 
 }  // namespace la

@@ -47,4 +47,17 @@ int launch_split_both(const SweepBoth& b, int dtype, hipStream_t st) {
     return LA_E_UNSUPPORTED;
 }
 
+// Every instantiation of this file made ready for its first launch on the current device.
+int prepare_split() {
+    int e = prep_family<__bf16, 192, 2, 1>();
+    if (!e) e = prep_family<__bf16, 192, 2, 2>();
+    if (!e) e = prep_family<__bf16, 256, 2, 1>();
+    if (!e) e = prep_family<__bf16, 256, 2, 2>();
+    if (!e) e = prep_family<_Float16, 192, 2, 1>();
+    if (!e) e = prep_family<_Float16, 192, 2, 2>();
+    if (!e) e = prep_family<_Float16, 256, 2, 1>();
+    if (!e) e = prep_family<_Float16, 256, 2, 2>();
+    return e;
+}
+
 }  // namespace la

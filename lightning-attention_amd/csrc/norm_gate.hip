@@ -330,20 +330,11 @@ static void ng_shape(int64_t chunks, bool backward, int* tpr, int* nv) {
     }
 }
 
-static int ng_cus() {
-    static const int cus = [] {
-        int dev = 0, n = 256;
-        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
-        return n > 0 ? n : 256;
-    }();
-    return cus;
-}
-
 // workgroups of a launch: enough to keep every CU's memory pipeline full, never more than row groups
 static int64_t ng_grid(int64_t rows, int tpr, bool backward) {
     const int64_t threads = ng_threads(tpr), rpg = threads / tpr, groups = (rows + rpg - 1) / rpg;
     if (!backward) return groups;  // nothing is carried from row to row: one group of rows per workgroup
-    const int64_t cap = 4 * (int64_t)ng_cus() * 256 / threads;  // ~16 wavefronts per CU
+    const int64_t cap = 4 * (int64_t)num_cus() * 256 / threads;  // ~16 wavefronts per CU
     return groups < cap ? groups : cap;
 }
 
@@ -406,6 +397,14 @@ static int ng_check(int64_t rows, int64_t cols, int dtype) {
     return norm_gate_supported(cols, dtype) ? LA_OK : LA_E_UNSUPPORTED;
 }
 
+}  // namespace la
+
+// Makes the runtime load this file's code object now (it otherwise does at the first launch from it).
+namespace la {
+int prepare_norm_gate() {
+    hipFuncAttributes attr;
+    return (int)hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(&norm_gate_reduce_kernel<float>));
+}
 }  // namespace la
 
 extern "C" int norm_gate_supported(int64_t cols, int dtype) {

@@ -228,6 +228,14 @@ static int launch_bwd(const void* x, const void* dy, const float* rstd, void* dx
 
 }  // namespace la
 
+// Makes the runtime load this file's code object now (it otherwise does at the first launch from it).
+namespace la {
+int prepare_srmsnorm() {
+    hipFuncAttributes attr;
+    return (int)hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(&srms_fwd_any<float>));
+}
+}  // namespace la
+
 extern "C" int srmsnorm_fwd(const void* x, void* y, float* rstd, int64_t rows, int64_t cols, int64_t row_stride,
                             float eps, int dtype, void* stream) {
     if (rows < 0 || cols <= 0 || row_stride < cols || rows > 0x7fffffffLL) return LA_E_SHAPE;

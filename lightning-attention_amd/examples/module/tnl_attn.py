@@ -47,9 +47,18 @@ class TnlAttention(nn.Module):
         mixed = lightning_attn_func(q, k, v, self.slope_rate)  # (b, h, n, d), token-major memory
         mixed = mixed.transpose(-3, -2).flatten(-2)            # (b, n, h*d): a view of that memory
         gate = self.output_gate(x)
-        if self.fused_norm_gate and mixed.is_cuda and norm_gate_supported(mixed.shape[-1], mixed.dtype):
+        if self._can_fuse(mixed, gate):
             return self.o_proj(norm_gate(mixed, gate, self.norm.weight, self.norm.bias, self.norm.eps))
         return self.o_proj(self.norm(mixed) * torch.sigmoid(gate))
+
+    def _can_fuse(self, mixed, gate):
+        """The fused kernel takes one dtype for the activations and the norm's parameters; anything else
+        (float32 LayerNorm parameters under autocast, a norm without bias, a width the kernel does not
+        take) goes through the three PyTorch operators, as in the reference."""
+        w, b = self.norm.weight, self.norm.bias
+        return (self.fused_norm_gate and mixed.is_cuda and w is not None and b is not None
+                and mixed.dtype == gate.dtype == w.dtype == b.dtype
+                and norm_gate_supported(mixed.shape[-1], mixed.dtype))
 
 
 if __name__ == "__main__":

@@ -16,7 +16,7 @@ LA_BF16, LA_FP16, LA_FP32 = 0, 1, 2
 _DTYPES = {torch.bfloat16: LA_BF16, torch.float16: LA_FP16, torch.float32: LA_FP32}
 
 SYMBOLS = (
-    "la_version", "la_error_string", "la_supported", "la_workspace_bytes",
+    "la_init", "la_version", "la_error_string", "la_supported", "la_workspace_bytes",
     "la_fwd", "la_bwd", "la_fwd_strided", "la_bwd_strided", "la_workspace_bytes_opts", "la_fwd_opts", "la_bwd_opts",
     "la_fwd_static", "la_saved_state_bytes", "la_saved_state_interval", "la_fwd_save", "la_bwd_saved",
     "srmsnorm_fwd", "srmsnorm_bwd", "norm_gate_supported", "norm_gate_workspace_bytes", "norm_gate_fwd", "norm_gate_bwd",
@@ -80,6 +80,8 @@ def lib():
                     "`python lightning-attention_amd/build.py`" % LIB_PATH
                 )
             L = ctypes.CDLL(LIB_PATH)
+            L.la_init.restype = _int
+            L.la_init.argtypes = []
             L.la_version.restype = ctypes.c_char_p
             L.la_version.argtypes = []
             L.la_error_string.restype = ctypes.c_char_p

@@ -7,18 +7,41 @@ import torch
 from . import _lib
 
 
+_supported = {}
+_ws_bytes = {}
+
+
 def norm_gate_supported(cols, dtype):
-    """True when the kernels take rows of `cols` elements of `dtype`."""
-    try:
-        code = _lib.dtype_code(dtype)
-    except TypeError:
-        return False
-    return bool(_lib.lib().norm_gate_supported(cols, code))
+    """True when the kernels take rows of `cols` elements of `dtype` (the answer depends on these two alone
+    and is remembered)."""
+    key = (cols, dtype)
+    got = _supported.get(key)
+    if got is None:
+        try:
+            got = bool(_lib.lib().norm_gate_supported(cols, _lib.dtype_code(dtype)))
+        except TypeError:
+            got = False
+        if len(_supported) > 1024:
+            _supported.clear()
+        _supported[key] = got
+    return got
+
+
+def _workspace_bytes(rows, cols, code):
+    key = (rows, cols, code)
+    got = _ws_bytes.get(key)
+    if got is None:
+        got = _lib.lib().norm_gate_workspace_bytes(rows, cols, code)
+        if len(_ws_bytes) > 1024:
+            _ws_bytes.clear()
+        _ws_bytes[key] = got
+    return got
 
 
 def _dense(t):
     """Row-major and 16-byte aligned (a dense view into a larger buffer may start off that grid)."""
-    t = t.contiguous()
+    if not t.is_contiguous():
+        t = t.contiguous()
     return t if t.data_ptr() % 16 == 0 else t.clone()
 
 
@@ -60,7 +83,7 @@ class _NormGate(torch.autograd.Function):
         dw, db = torch.empty_like(weight), torch.empty_like(bias)
         L = _lib.lib()
         with _lib.on_device(o2.device):
-            ws_bytes = L.norm_gate_workspace_bytes(rows, cols, code)
+            ws_bytes = _workspace_bytes(rows, cols, code)
             ws = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=o2.device)
             rc = L.norm_gate_bwd(o2.data_ptr(), g2.data_ptr(), weight.data_ptr(), bias.data_ptr(), mean.data_ptr(),
                                  rstd.data_ptr(), dy2.data_ptr(), d_o.data_ptr(), d_g.data_ptr(), dw.data_ptr(), db.data_ptr(),

@@ -62,3 +62,28 @@ def test_state_dict_names_follow_the_reference():
     assert names == {"q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight", "norm.weight", "norm.bias",
                      "output_gate.0.weight", "output_gate.1.weight"}
     assert block.slope_rate.shape == (4, 1, 1)
+
+
+def test_float32_norm_parameters_take_the_unfused_path():
+    """A LayerNorm kept in float32 beside bf16 activations (master weights, autocast) cannot go through the fused
+    kernel, which takes one dtype: the block then runs the three PyTorch operators of tnl_attn.py:66-69 instead
+    of raising, and agrees with the fused path on bf16 parameters to bf16 rounding."""
+    torch.manual_seed(4)
+    block = tnl.TnlAttention(512, 4).cuda().bfloat16()
+    x = torch.randn(2, 200, 512, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        fused = block(x)
+    block.norm.float()
+    gate = block.output_gate(x)
+    assert not block._can_fuse(x, gate)
+    with torch.autocast("cuda", dtype=torch.bfloat16), torch.no_grad():
+        y = block(x)
+    torch.cuda.synchronize()
+    assert y.shape == fused.shape
+    assert rel_norm(y.float(), fused.float()) < 2e-2
+    # a norm without bias is not the fused kernel's either
+    block2 = tnl.TnlAttention(512, 4).cuda().bfloat16()
+    block2.norm = torch.nn.LayerNorm(512, bias=False).cuda().bfloat16()
+    assert not block2._can_fuse(x, gate)
+    with torch.no_grad():
+        assert block2(x).shape == x.shape

@@ -60,6 +60,22 @@ def test_static_scratch_forward_matches_workspace_forward():
         got = _la_fwd_static(L, q, k, v, s)
         results.append((q, k, v, s, need, got))
     torch.cuda.synchronize()
+    # the property the entry point exists for: a call allocates no device memory (the outputs are
+    # made first; the first calls above have looked the array's address up already)
+    outs = [torch.full_like(v, float("nan")) for (_, _, v, _, _, _) in results]
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    reserved0 = torch.cuda.memory_reserved()
+    st = torch.cuda.current_stream().cuda_stream
+    for (q, k, v, s, _, _), o in zip(results, outs):
+        b, h, n, d = q.shape
+        rc = L.la_fwd_static(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr() if s is not None else None,
+                             o.data_ptr(), b, h, n, d, v.shape[-1], 0, st)
+        assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0 and torch.cuda.memory_reserved() == reserved0
+    for (_, _, _, _, _, got), o in zip(results, outs):
+        assert torch.equal(got, o)
     for q, k, v, s, need, got in results:
         want = _la_fwd(L, q, k, v, s, need)
         torch.cuda.synchronize()
