@@ -11,7 +11,9 @@ MFMA rate of the step (flop count of a 64-token block recurrence, 344064 flop pe
 token and head, divided by the measured time); ``ms_per_step`` is the same
 measurement in milliseconds: W untimed warm-up steps, then exactly K steps between two
 device synchronisations on the host clock.  The same K steps are also bracketed one by
-one with HIP events (``step_event_ms``: median, min, mean).
+one with HIP events (``step_event_ms``: median, min, mean).  ``roofline.traffic`` comes from a committed
+rocprofv3 counter summary and is withheld when the kernel sources have changed since it was taken;
+``parity.literal_fail_frac`` states how often the step's own results miss the tolerance as literally named.
 
 The secondary measurements (fwd / bwd split, n sweep, other configurations, SRMSNorm and,
 last, the per-launch roofline figures of the step's own kernels) run BEFORE the headline
@@ -227,14 +229,59 @@ def cpu_baseline_srmsnorm(rows=32768, cols=4096):
             "bwd_GBps": round(bb / (statistics.median(bwd) * 1e-3) / 1e9, 2)}
 
 
+def kernel_sources_sha16():
+    """First 16 hex digits of the SHA-256 over the library's sources (csrc/*.hip, *.h and the public header), in
+    name order: what the committed counter summary is tied to."""
+    import glob
+    import hashlib
+
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "lightning-attention_amd", "csrc")
+    files = sorted(glob.glob(os.path.join(csrc, "*.hip")) + glob.glob(os.path.join(csrc, "*.h")))
+    files.append(os.path.join(ROOT, "include", "lightning_attn_hip.h"))
+    for path in files:
+        with open(path, "rb") as f:
+            h.update(os.path.basename(path).encode() + b"\0" + f.read())
+    return h.hexdigest()[:16]
+
+
 def counter_traffic():
-    """HBM bytes per launch from the committed rocprofv3 counter summary (bench.py cannot read
-    hardware counters itself); {} when the file is absent."""
+    """HBM bytes per launch from the committed rocprofv3 counter summary (bench.py cannot read hardware counters
+    itself).  The summary names the kernel sources it was taken with; when they are not the ones in this tree the
+    figures are withheld.  Returns (summary, reason for withholding or None)."""
     try:
         with open(TRAFFIC_JSON) as f:
-            return json.load(f)
+            data = json.load(f)
     except (OSError, ValueError):
-        return {}
+        return {}, "no counter summary at profiles/%s" % os.path.basename(TRAFFIC_JSON)
+    have, want = data.get("kernel_sources_sha16"), kernel_sources_sha16()
+    if have != want:
+        return {}, ("the counter summary was taken with other kernel sources (%s, this tree %s): profile again with "
+                    "benchmarks/profile_summary.py" % (have, want))
+    return data, None
+
+
+def literal_tolerance(got, q, k, v, s_head, do):
+    """Share of elements outside the tolerance as literally stated, |a - ref| <= 2e-2 + 2e-2 |ref|, for one (batch,
+    head) sequence of the workload: the HIP results `got` = (o, dq, dk, dv) and the reference's own naive path run in
+    bf16 (the oracle's restatement of linear_attention.py:27-34, same rounding order), both against the naive path in
+    float32 on the same bf16-rounded inputs.  With N(0,1) inputs the outputs have an RMS of 10..100, so the absolute
+    term is a fraction of a bf16 ulp and no bf16 pipeline can meet the bound on every element; the parity tests scale
+    the absolute term by the RMS of the expected values and assert that the kernels miss the literal bound no more
+    often than the reference's dataflow does."""
+    import torch
+
+    import oracle
+
+    truth = oracle.linear_attn_fwd_bwd(q.float(), k.float(), v.float(), s_head, do.float(), torch.float32)
+    ref16 = oracle.linear_attn_fwd_bwd(q, k, v, s_head, do, None)
+    res = {}
+    for name, a, r16, t in zip(("o", "dq", "dk", "dv"), got, ref16, truth):
+        bound = 2e-2 + 2e-2 * t.abs()
+        res[name] = {"hip": round(((a.float() - t).abs() > bound).float().mean().item(), 5),
+                     "reference_bf16_dataflow": round(((r16.float() - t).abs() > bound).float().mean().item(), 5),
+                     "hip_rel_frobenius": round(((a.float() - t).norm() / t.norm()).item(), 5)}
+    return res
 
 
 def main():
@@ -391,10 +438,22 @@ def main():
     if q is None or q.shape != (B, H, N, D):
         q = k = v = do = None
         q, k, v, do = inputs(N)
+    # one sequence of the workload, as the step's own launches compute it, for the literal-tolerance figures
+    HEAD_SAMPLE = 16
+    o = lightning_attn_func(q, k, v, s)
+    o.backward(do)
+    torch.cuda.synchronize()
+    sample = tuple(t[0:1, HEAD_SAMPLE:HEAD_SAMPLE + 1].detach().cpu() for t in (o, q.grad, k.grad, v.grad))
+    sample_in = tuple(t[0:1, HEAD_SAMPLE:HEAD_SAMPLE + 1].detach().cpu() for t in (q, k, v, do))
+    del o
+    q.grad = k.grad = v.grad = None
+
     # ---- per-launch figures: direct calls of the C entry points, HIP events on the launch stream ----
-    counters = counter_traffic()
+    counters, counters_withheld = counter_traffic()
     buf = [torch.empty_like(v) for _ in range(3)]
     qd, kd, vd = q.detach(), k.detach(), v.detach()
+    sv_bytes = L.la_saved_state_bytes(B, H, N, D, D, 0, None)
+    saved = torch.empty(max(sv_bytes, 4) // 4, dtype=torch.float32, device=dev)
 
     def fwd_launch():  # O = sweep(Q, K, V)
         rc = L.la_fwd(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), s.data_ptr(), buf[0].data_ptr(), B, H, N, D, D, 0, None, 0, st)
@@ -409,6 +468,17 @@ def main():
                       buf[1].data_ptr(), buf[2].data_ptr(), B, H, N, D, D, 0, None, 0, st)
         assert rc == 0, rc
 
+    def fwd_save_launch():  # the forward launch as the operator runs it when a backward pass will follow
+        rc = L.la_fwd_save(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), s.data_ptr(), buf[0].data_ptr(), None, B, H, N, D, D, 0,
+                           None, 0, None, saved.data_ptr(), sv_bytes, st)
+        assert rc == 0, rc
+
+    def bwd_saved_launches():  # dQ in chunks from the saved states (128-column workgroups), then dK and dV
+        rc = L.la_bwd_saved(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), s.data_ptr(), do.data_ptr(), buf[0].data_ptr(),
+                            buf[1].data_ptr(), buf[2].data_ptr(), None, B, H, N, D, D, 0, None, 0, None,
+                            saved.data_ptr(), sv_bytes, st)
+        assert rc == 0, rc
+
     def launch_entry(kernel, what, ts, nbytes, nflop, counter_key):
         med = statistics.median(ts)
         c = counters.get(counter_key) or {}
@@ -420,6 +490,7 @@ def main():
             # counter reads for a cast kernel of known size (profiles/, written by benchmarks/profile_summary.py)
             "traffic": c.get("hbm_bytes"),
             "traffic_source": ("profiles/%s" % os.path.basename(TRAFFIC_JSON)) if c else None,
+            "traffic_withheld": None if c else (counters_withheld or "no entry %r in the counter summary" % counter_key),
             "algorithmic_bytes": nbytes, "launch_ms": stats(ts),
             "mfma_tflops": round(nflop / (med * 1e-3) / 1e12, 1),
             "mfma_frac": round(nflop / (med * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
@@ -429,19 +500,33 @@ def main():
     dq_ts = event_times_timed(dq_launch)
     bwd_ts = event_times_timed(bwd_launches)
     pair_ts = [max(b_ - statistics.median(dq_ts), 1e-6) for b_ in bwd_ts]
+    fwd_save_launch()
+    fwd_save_ts = event_times_timed(fwd_save_launch)
+    bwd_saved_ts = event_times_timed(bwd_saved_launches)
+    dq_resumed_ts = [max(b_ - statistics.median(pair_ts), 1e-6) for b_ in bwd_saved_ts]
     fb, ff = bytes_per_token(D, D, "fwd") * tokens, flops_per_token(D, D, "fwd") * tokens
     pair_bytes = 6 * D * 2 * tokens  # q, k, v, dO read once; dK, dV written once
     pair_flop = flops_per_token(D, D, "bwd") * tokens - ff
     roofline = launch_entry("la_sweep_pipe_kernel<bf16, DKP=128, 64 columns, forward, decay>",
-                            "O = sweep(Q,K,V); a step is this, the same for dQ, and one launch for dK + dV",
-                            fwd_ts, fb, ff, "forward")
+                            "O = sweep(Q,K,V) with the state left at the chunk boundary (la_fwd_save); a step is this, "
+                            "a launch for dQ and one for dK + dV",
+                            fwd_save_ts, fb, ff, "forward")
     other_launches = [
-        launch_entry("la_sweep_pipe_kernel<bf16, DKP=128, 64 columns, forward, decay>", "dQ = sweep(dO,V,K)", dq_ts, fb, ff, "forward"),
+        launch_entry("la_sweep_pipe_kernel<bf16, DKP=128, 128 columns, forward, decay>",
+                     "dQ = sweep(dO,V,K) in two chunks per sequence from the saved states (la_bwd_saved minus the dK + dV launch)",
+                     dq_resumed_ts, fb, ff, "forward_wide"),
         launch_entry("la_sweep_pipe_kernel<bf16, DKP=128, 128 columns, reverse, decay>",
                      "dK + dV in one launch (la_bwd minus the dQ launch, gap between the two included)",
                      pair_ts, pair_bytes, pair_flop, "reverse_pair"),
+        launch_entry("la_sweep_pipe_kernel<bf16, DKP=128, 64 columns, forward, decay>",
+                     "not part of the step: O = sweep(Q,K,V) without saving (la_fwd)", fwd_ts, fb, ff, "forward"),
+        launch_entry("la_sweep_pipe_kernel<bf16, DKP=128, 64 columns, forward, decay>",
+                     "not part of the step: dQ = sweep(dO,V,K) recomputing its state (la_bwd's dQ launch without saved states)",
+                     dq_ts, fb, ff, "forward"),
     ]
-    buf = None
+    direct_ms = {"la_fwd_save": stats(fwd_save_ts), "la_bwd_saved": stats(bwd_saved_ts),
+                 "la_fwd": stats(fwd_ts), "la_bwd": stats(bwd_ts)}
+    buf = saved = None
 
     # ---- the headline region -------------------------------------------------------------------------
     ms, ev_ts = timed_steps(step, args.warmup, args.steps)
@@ -469,10 +554,19 @@ def main():
         "step_hbm_frac": round(bytes_step / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
         "roofline": roofline,
         "roofline_other_launches": other_launches,
+        "entry_points_ms": direct_ms,
     }
     line.update(out)
 
     if not args.no_cpu:
+        # (CPU leg: the oracle as checker and as baseline)
+        line["parity"] = {
+            "tolerance_asserted_in_tests": "|a - ref| <= 2e-2 max(1, rms_seq(ref)) + 2e-2 |ref| element-wise and relative "
+                                           "Frobenius error < 1e-2 (bf16); relative error < 1e-4 (fp32)",
+            "literal_fail_frac": literal_tolerance(sample, *sample_in[:3], s[HEAD_SAMPLE:HEAD_SAMPLE + 1].cpu(), sample_in[3]),
+            "literal_fail_frac_sample": "batch 0, head %d of the step's own results; share of elements with "
+                                        "|a - ref| > 2e-2 + 2e-2 |ref| against the float32 naive path" % HEAD_SAMPLE,
+        }
         line["cpu_baseline"] = cpu_baseline()
         line["cpu_baseline_config1"] = cpu_baseline_config1()
         line["cpu_baseline_srmsnorm"] = cpu_baseline_srmsnorm()

@@ -30,20 +30,17 @@ def classify(name):
     """Short key of a kernel this repository launches (or of the calibration cast), None for others."""
     if "bfloat16_copy_kernel" in name:
         return "cast_f32_to_bf16"
+    if "la_sweep_pipe_both_kernel" in name:
+        return "sweep_both"
     if "la_sweep_pipe_kernel" in name:
-        m = re.search(r"Li(\d+)ELi(\d)ELb(\d)E", name) or re.search(r"<[^,]+, *(\d+), *(\d), *(true|false|0|1)", name)
+        # la_sweep_pipe_kernel<T, DKP, NF, NH, REVERSE, DECAY, DENSE>, mangled or demangled
+        m = (re.search(r"Li(\d+)ELi(\d)ELi(\d)ELb(\d)E", name)
+             or re.search(r"<[^,]+, *(\d+), *(\d), *(\d), *(true|false|0|1)", name))
         if not m:
             return "sweep_pipe"
-        rev = m.group(3) in ("1", "true")
-        wide = m.group(2) == "2"
-        return ("reverse" if rev else "forward") + ("_pair" if rev and wide else "_wide" if wide else "")
-    if "la_sweep_wide_kernel" in name:
-        m = re.search(r"Li(\d+)ELb(\d)E", name) or re.search(r"<[^,]+, *(\d+), *(true|false|0|1)", name)
-        return "sweep_wide%s_%s" % (m.group(1), "reverse" if m.group(2) in ("1", "true") else "forward") if m else "sweep_wide"
-    if "la_sweep_both_kernel" in name or "la_sweep_pipe_both_kernel" in name:
-        return "sweep_both"
-    if "la_sweep_kernel" in name:
-        return "sweep_classic"
+        dkp, rev, wide = int(m.group(1)), m.group(4) in ("1", "true"), m.group(3) == "2"
+        key = ("reverse" if rev else "forward") + ("_pair" if rev and wide else "_wide" if wide else "")
+        return key if dkp <= 128 else "d%d_%s" % (dkp, key)
     if "la_state_scan" in name:
         return "state_scan"
     if "norm_gate_fwd" in name:
@@ -86,6 +83,17 @@ def durations(folder):
                 "median_us": round(statistics.median(v), 1), "max_us": round(max(v), 1)} for k, v in vals.items()}
 
 
+def kernel_names(folder):
+    """The kernel names behind each key, as the trace spells them."""
+    names = collections.defaultdict(set)
+    for path in glob.glob(os.path.join(folder, "**", "*kernel_trace.csv"), recursive=True):
+        for r in csv.DictReader(open(path)):
+            key = classify(r["Kernel_Name"])
+            if key:
+                names[key].add(r["Kernel_Name"])
+    return {k: sorted(v) for k, v in names.items()}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--kt")
@@ -93,6 +101,7 @@ def main():
     ap.add_argument("--write")
     ap.add_argument("--out", required=True)
     ap.add_argument("--cast-elements", type=int, default=CAST_ELEMENTS)
+    ap.add_argument("--git-head", default=None, help="commit the run was made at (the GPU box holds no .git)")
     a = ap.parse_args()
     cast_read, cast_write = 4 * a.cast_elements, 2 * a.cast_elements
     res = collections.defaultdict(dict)
@@ -113,6 +122,30 @@ def main():
             rd, wr = fetch[k] * 1024.0 * fs, write[k] * 1024.0 * ws
             res[k].update({"FETCH_SIZE_KiB": round(fetch[k], 1), "WRITE_SIZE_KiB": round(write[k], 1),
                            "read_bytes": round(rd), "write_bytes": round(wr), "hbm_bytes": round(rd + wr), "dispatches": nf[k]})
+    # what the figures are tied to: the kernel sources (bench.py withholds the traffic figures when they change),
+    # the commit and the day
+    import datetime
+    import hashlib
+    import subprocess
+
+    here = os.path.dirname(os.path.abspath(__file__))
+    root = os.path.dirname(os.path.dirname(here))
+    h = hashlib.sha256()
+    csrc = os.path.join(os.path.dirname(here), "csrc")
+    files = sorted(glob.glob(os.path.join(csrc, "*.hip")) + glob.glob(os.path.join(csrc, "*.h")))
+    files.append(os.path.join(root, "include", "lightning_attn_hip.h"))
+    for path in files:
+        with open(path, "rb") as f:
+            h.update(os.path.basename(path).encode() + b"\0" + f.read())
+    res["kernel_sources_sha16"] = h.hexdigest()[:16]
+    res["git_head"] = a.git_head
+    if not res["git_head"]:
+        try:
+            res["git_head"] = subprocess.run(["git", "-C", root, "rev-parse", "HEAD"], capture_output=True, text=True).stdout.strip() or None
+        except OSError:
+            res["git_head"] = None
+    res["date"] = datetime.date.today().isoformat()
+    res["kernels"] = kernel_names(a.kt) if a.kt else {}
     with open(a.out, "w") as f:
         json.dump(res, f, indent=1, sort_keys=True)
         f.write("\n")
