@@ -162,6 +162,21 @@ int la_bwd_opts(const void *q, const void *k, const void *v, const float *s, con
                 void *workspace, size_t ws_bytes, const la_launch_opts *opts, void *stream);
 
 /*
+ * la_fwd_opts on pre-activations: O = attention(silu(q), silu(k), silu(v)), silu(t) = t / (1 + exp(-t))
+ * evaluated in float32 and rounded to the tensors' type where the tiles are loaded, so that the activated
+ * tensors never exist in memory.  This is the forward pass of the reference's attention block without its
+ * three activation passes (`F.silu(self.q_proj(x))` ..., examples/module/tnl_attn.py:51-54) for callers that
+ * need no backward pass (inference): 0.36 against 0.56 ms at b4 h32 n8192 d=e=128.  bf16 / fp16 with
+ * d, e <= 128 (la_fwd_silu_supported; LA_E_UNSUPPORTED otherwise: apply the activation first and call la_fwd).
+ * Workspace as for la_fwd.
+ */
+int la_fwd_silu_supported(int64_t d, int64_t e, int dtype);
+int la_fwd_silu(const void *q, const void *k, const void *v, const float *s, void *o,
+                const int64_t *strides,
+                int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype,
+                void *workspace, size_t ws_bytes, const la_launch_opts *opts, void *stream);
+
+/*
  * Forward and backward pass as a pair: the forward pass leaves its d x e float state K^T V at a few
  * token boundaries, and the dQ sweep of the backward pass - whose state V^T K is the transpose - starts
  * one chunk of each sequence at each of them.  It then needs neither warm-up blocks nor collect and scan

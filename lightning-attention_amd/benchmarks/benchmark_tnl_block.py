@@ -35,7 +35,7 @@ def main():
     if "--large" in sys.argv:  # the block around the benchmark shape of the operator only
         shapes = shapes[-1:]
     print("TNL block, bf16: b, n, embed, heads | block fwd+bwd ms, fused norm-gate / separate operators | "
-          "norm-gate alone fwd, bwd ms: fused / separate")
+          "norm-gate alone fwd, bwd ms: fused / separate | block forward without gradients, SiLU in the kernel / separate")
     for b, n, embed, heads in shapes:
         block = tnl.TnlAttention(embed, heads).to(dev).bfloat16()
         x = torch.randn(b, n, embed, device=dev, dtype=torch.bfloat16).requires_grad_()
@@ -49,6 +49,14 @@ def main():
         for fused in (True, False):
             block.fused_norm_gate = fused
             times[fused] = do_bench(step, grads=params)
+        # inference: the forward pass alone without gradients, SiLU inside the forward kernel / as three PyTorch passes
+        infer = {}
+        block.fused_norm_gate = True
+        for fused in (True, False):
+            block.fused_silu = fused
+            with torch.no_grad():
+                infer[fused] = do_bench(lambda: block(x))
+        block.fused_silu = True
         # the norm / gate part on its own
         o, gate = (torch.randn(b * n, embed, device=dev, dtype=torch.bfloat16).requires_grad_() for _ in range(2))
         w, bias = block.norm.weight, block.norm.bias
@@ -59,9 +67,9 @@ def main():
             y = fn()
             parts[name] = (do_bench(fn), do_bench(lambda: y.backward(dy, retain_graph=True), grads=(o, gate, w, bias)))
             del y
-        print("%d %5d %5d %3d | %.4f / %.4f | fwd %.4f / %.4f  bwd %.4f / %.4f"
+        print("%d %5d %5d %3d | %.4f / %.4f | fwd %.4f / %.4f  bwd %.4f / %.4f | inference fwd, SiLU fused / separate %.4f / %.4f"
               % (b, n, embed, heads, times[True], times[False], parts["fused"][0], parts["separate"][0],
-                 parts["fused"][1], parts["separate"][1]), flush=True)
+                 parts["fused"][1], parts["separate"][1], infer[True], infer[False]), flush=True)
         del block, x, g, o, gate, dy
 
 

@@ -7,6 +7,8 @@
 namespace la {
 int sweep(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
           bool reverse, void* ws, size_t ws_bytes, const Opts& opts, hipStream_t st);
+int sweep_silu(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
+               void* ws, size_t ws_bytes, const Opts& opts, hipStream_t st);
 int sweep_bwd_once(const SweepIO& dq, const SweepIO& dk, const SweepIO& dv, const float* s, int64_t bh, int64_t h, int64_t n,
                    int64_t d, int dtype, void* ws, size_t ws_bytes, const Opts& opts, hipStream_t st);
 int sweep_fwd_rev_once(const SweepIO& fwd, const SweepIO& rev, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk,
@@ -101,7 +103,8 @@ static bool saved_usable(const Saved& sv, const SavedPlan& pl) {
 }
 
 static int fwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s, const Tensor& o, int64_t b, int64_t h,
-               int64_t n, int64_t d, int64_t e, int dtype, const Scratch& ws, const Opts& opts, const Saved& sv, hipStream_t st) {
+               int64_t n, int64_t d, int64_t e, int dtype, const Scratch& ws, const Opts& opts, const Saved& sv, hipStream_t st,
+               bool silu = false) {
     int rc = check_dims(b, h, n, d, e, dtype);
     if (rc != LA_OK) return rc;
     if ((rc = check_opts(opts)) != LA_OK) return rc;
@@ -112,6 +115,7 @@ static int fwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s
         if (!ts[i]->p) return LA_E_NULLPTR;
     for (int i = 0; i < 4; ++i)
         if ((rc = check_tensor(*ts[i], b, h, n, cols[i], dtype)) != LA_OK) return rc;
+    if (silu) return sweep_silu(io(q, k, v, o), s, b * h, h, n, d, e, dtype, ws.p, ws.bytes, opts, st);
     if (sv.p) {
         const SavedPlan pl = plan_saved(b * h, n, d, e, dtype, opts);
         if (saved_usable(sv, pl)) return sweep_saving(io(q, k, v, o), s, b * h, h, n, d, e, dtype, sv.p, pl.chunk_len, st);
@@ -226,6 +230,26 @@ extern "C" int la_fwd_save(const void* q, const void* k, const void* v, const fl
         return la::fwd(dense(q, h, n, d), dense(k, h, n, d), dense(v, h, n, e), s, dense(o, h, n, e), b, h, n, d, e, dtype, ws, op, sv, st);
     return la::fwd(strided(q, strides), strided(k, strides + 3), strided(v, strides + 6), s, strided(o, strides + 9), b, h, n,
                    d, e, dtype, ws, op, sv, st);
+}
+
+extern "C" int la_fwd_silu_supported(int64_t d, int64_t e, int dtype) {
+    return (dtype == LA_BF16 || dtype == LA_FP16) && d <= 128 && e <= 128 && la_supported(d, e, dtype);
+}
+
+extern "C" int la_fwd_silu(const void* q, const void* k, const void* v, const float* s, void* o, const int64_t* strides,
+                           int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype, void* workspace,
+                           size_t ws_bytes, const la_launch_opts* opts, void* stream) {
+    if (la_supported(d, e, dtype) && !la_fwd_silu_supported(d, e, dtype)) return LA_E_UNSUPPORTED;
+    const la::Scratch ws = {workspace, workspace ? ws_bytes : 0};
+    const la::Saved none = {nullptr, 0};
+    const la::Opts& op = opts ? *opts : la::kAuto;
+    const hipStream_t st = static_cast<hipStream_t>(stream);
+    using la::dense;
+    using la::strided;
+    if (!strides)
+        return la::fwd(dense(q, h, n, d), dense(k, h, n, d), dense(v, h, n, e), s, dense(o, h, n, e), b, h, n, d, e, dtype, ws, op, none, st, true);
+    return la::fwd(strided(q, strides), strided(k, strides + 3), strided(v, strides + 6), s, strided(o, strides + 9), b, h, n,
+                   d, e, dtype, ws, op, none, st, true);
 }
 
 extern "C" int la_fwd_opts(const void* q, const void* k, const void* v, const float* s, void* o, const int64_t* strides,

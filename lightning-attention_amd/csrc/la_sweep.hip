@@ -214,6 +214,17 @@ int sweep(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, i
     return launch_planned(p, bh, n, dk, dv, dtype, reverse, ws, ws_bytes, opts, st);
 }
 
+// The forward sweep over silu(x), silu(y), silu(z): the same plan, the activation applied in the tile load.
+int sweep_silu(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
+               void* ws, size_t ws_bytes, const Opts& opts, hipStream_t st) {
+    if (dk > 128 || dv > 128 || (dtype != LA_BF16 && dtype != LA_FP16)) return LA_E_UNSUPPORTED;
+    SweepPair p;
+    p.nprod = 1;
+    p.silu = 1;
+    p.a[0] = make_args(io, s, bh, h, n, dk, dv);
+    return launch_planned(p, bh, n, dk, dv, dtype, false, ws, ws_bytes, opts, st);
+}
+
 // States a forward sweep can leave behind for the sweep that follows it over the same tensors in swapped roles.
 // O = sweep(q, k, v) carries the state K^T V (d x e); dQ = sweep(dO, v, k) of the backward pass carries V^T K,
 // its transpose.  Where the forward pass walks each sequence in one piece and leaves the state at c - 1

@@ -126,6 +126,9 @@ struct SweepPair {
     // nullptr / 0: nothing is saved.
     float* save = nullptr;
     int save_len = 0;
+    // x, y and z are pre-activations: the kernel applies SiLU to them as it loads them (forward sweeps of
+    // the pipelined kernel at feature dims up to 128)
+    int silu = 0;
 };
 
 // One launch can also carry sweeps of both directions: the whole backward pass when d == e, dQ walking

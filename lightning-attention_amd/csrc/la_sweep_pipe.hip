@@ -12,6 +12,18 @@ static int launch_dir(const SweepPair& pair, hipStream_t st) {
     const bool dense = all_plain(pair);
 #define LA_GO2(DKP, NH, DENSE) (decay ? launch_one<T, DKP, 1, NH, REVERSE, true, DENSE>(pair, st) : launch_one<T, DKP, 1, NH, REVERSE, false, DENSE>(pair, st))
 #define LA_GO(DKP, NH) (dense ? LA_GO2(DKP, NH, true) : LA_GO2(DKP, NH, false))
+    if (pair.silu) {
+        if constexpr (!REVERSE) {
+#define LA_GS2(DKP, NH, DENSE) (decay ? launch_one<T, DKP, 1, NH, false, true, DENSE, true>(pair, st) : launch_one<T, DKP, 1, NH, false, false, DENSE, true>(pair, st))
+#define LA_GS(DKP, NH) (dense ? LA_GS2(DKP, NH, true) : LA_GS2(DKP, NH, false))
+            if (pair.wide) return LA_GS(128, 2);
+            if (a.dk <= 64) return LA_GS(64, 1);
+            return LA_GS(128, 1);
+#undef LA_GS
+#undef LA_GS2
+        }
+        return LA_E_UNSUPPORTED;
+    }
     if (pair.wide) return LA_GO(128, 2);  // 128 columns per workgroup (nslice counts those)
     if (a.dk <= 64) return LA_GO(64, 1);
     return LA_GO(128, 1);
@@ -83,6 +95,7 @@ int launch_state_scan(const SweepPair& p, hipStream_t st) {
 }
 
 static int launch_any(const SweepPair& p, int dtype, bool reverse, hipStream_t st) {
+    if (p.silu && (p.a[0].dk > 128 || reverse || p.nprod != 1)) return LA_E_UNSUPPORTED;
     if (p.a[0].dk > 128) return launch_split(p, dtype, reverse, st);
     if (dtype == LA_BF16) return reverse ? launch_dir<__bf16, true>(p, st) : launch_dir<__bf16, false>(p, st);
     if (dtype == LA_FP16) return reverse ? launch_dir<_Float16, true>(p, st) : launch_dir<_Float16, false>(p, st);
@@ -97,6 +110,14 @@ int prepare_pipe() {
     if (!e) e = prep_family<_Float16, 64, 1, 1>();
     if (!e) e = prep_family<_Float16, 128, 1, 1>();
     if (!e) e = prep_family<_Float16, 128, 1, 2>();
+#define LA_PS(T, DKP, NH) \
+    if (!e) e = prep_one<T, DKP, 1, NH, false, false, false, true>(); \
+    if (!e) e = prep_one<T, DKP, 1, NH, false, false, true, true>();  \
+    if (!e) e = prep_one<T, DKP, 1, NH, false, true, false, true>();  \
+    if (!e) e = prep_one<T, DKP, 1, NH, false, true, true, true>();
+    LA_PS(__bf16, 64, 1) LA_PS(__bf16, 128, 1) LA_PS(__bf16, 128, 2)
+    LA_PS(_Float16, 64, 1) LA_PS(_Float16, 128, 1) LA_PS(_Float16, 128, 2)
+#undef LA_PS
     if (!e) e = prepare_split();
     return e;
 }

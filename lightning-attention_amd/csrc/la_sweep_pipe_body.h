@@ -61,7 +61,9 @@ struct PipeLds {
 // DENSE: all four tensors are plain (b, h, n, d) arrays; their rows then take a shorter addressing path
 // (see load_step).
 // `bid`: number of the workgroup within its part of the launch.
-template <typename T, int DKP, int NF, int NH, bool REVERSE, bool DECAY, bool DENSE>
+// SILU: x, y and z pass through SiLU on their way from memory into LDS (the attention block's activation on
+// q, k, v, examples/module/tnl_attn.py:51-54, fused into the forward pass).
+template <typename T, int DKP, int NF, int NH, bool REVERSE, bool DECAY, bool DENSE, bool SILU = false>
 __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const unsigned bid) {
     typedef Mma<T> M;
     typedef typename M::V8 V8;
@@ -318,6 +320,17 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
     };
     auto stage_step = [&](auto hc, int buf, int zslot, const u32x4 (&xr)[XC], const u32x4 (&yr)[XC], const u32x4 (&zr)[ZC], int64_t bout, bool flush) __attribute__((always_inline)) {
         constexpr int HC = decltype(hc)::value;
+        // SILU: silu(t) = t / (1 + exp(-t)) in float32, rounded back to the tensors' type; padding stays zero
+        auto silu16 = [](u32x4 v) {
+            typedef T T8 __attribute__((ext_vector_type(8)));
+            T8 t = __builtin_bit_cast(T8, v);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float f = (float)t[i];
+                t[i] = (T)(f * __builtin_amdgcn_rcpf(1.f + __expf(-f)));
+            }
+            return __builtin_bit_cast(u32x4, t);
+        };
         const unsigned xd = opaque(buf * XYB + (ROWAL ? lane_stage_xy : 0u));
         const unsigned zd = opaque(ZBASE + zslot * ZTB + lane_stage_z);
         u32x4 o[ZC];
@@ -329,19 +342,19 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
         for (int u = 0; u < XC; ++u) {
             if constexpr (ROWAL) {
                 // chunk c = tid + NL u lies CROWS rows below chunk tid
-                *reinterpret_cast<u32x4*>(smem + xd + u * CROWS * XS * E) = xr[u];
-                *reinterpret_cast<u32x4*>(smem + xd + YOFF + u * CROWS * XS * E) = yr[u];
+                *reinterpret_cast<u32x4*>(smem + xd + u * CROWS * XS * E) = SILU ? silu16(xr[u]) : xr[u];
+                *reinterpret_cast<u32x4*>(smem + xd + YOFF + u * CROWS * XS * E) = SILU ? silu16(yr[u]) : yr[u];
             } else {
                 const int c = tid + NL * u;
                 const unsigned so = xd + ((c / CPX) * XS + (c % CPX) * 8) * E;
-                *reinterpret_cast<u32x4*>(smem + so) = xr[u];
-                *reinterpret_cast<u32x4*>(smem + so + YOFF) = yr[u];
+                *reinterpret_cast<u32x4*>(smem + so) = SILU ? silu16(xr[u]) : xr[u];
+                *reinterpret_cast<u32x4*>(smem + so + YOFF) = SILU ? silu16(yr[u]) : yr[u];
             }
         }
         if constexpr (HC == 0) {
             store_out(bout, flush, o);
 #pragma unroll
-            for (int u = 0; u < ZC; ++u) *reinterpret_cast<u32x4*>(smem + zd + u * ZROWS * ZS * E) = zr[u];
+            for (int u = 0; u < ZC; ++u) *reinterpret_cast<u32x4*>(smem + zd + u * ZROWS * ZS * E) = SILU ? silu16(zr[u]) : zr[u];
         }
     };
 
@@ -728,9 +741,9 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
     }
 }
 
-template <typename T, int DKP, int NF, int NH, bool REVERSE, bool DECAY, bool DENSE>
+template <typename T, int DKP, int NF, int NH, bool REVERSE, bool DECAY, bool DENSE, bool SILU = false>
 __global__ __launch_bounds__(512, 1) void la_sweep_pipe_kernel(SweepPair pair) {
-    sweep_pipe_body<T, DKP, NF, NH, REVERSE, DECAY, DENSE>(pair, blockIdx.x);
+    sweep_pipe_body<T, DKP, NF, NH, REVERSE, DECAY, DENSE, SILU>(pair, blockIdx.x);
 }
 
 // Forward-walking and backward-walking sweeps in one launch (SweepBoth).
@@ -741,20 +754,21 @@ __global__ __launch_bounds__(512, 1) void la_sweep_pipe_both_kernel(SweepBoth bo
 }
 
 // What a kernel instantiation needs once per device before its first launch (its dynamic LDS limit raised).
-template <typename T, int DKP, int NF, int NH, bool REVERSE, bool DECAY, bool DENSE>
+template <typename T, int DKP, int NF, int NH, bool REVERSE, bool DECAY, bool DENSE, bool SILU = false>
 static int prep_one() {
     constexpr size_t lds = PipeLds<DKP, NF, NH>::bytes(sizeof(T));
     static_assert(lds <= 160 * 1024, "LDS budget");
     static unsigned char lds_allowed[kMaxDevices];
-    return allow_lds(la_sweep_pipe_kernel<T, DKP, NF, NH, REVERSE, DECAY, DENSE>, lds, lds_allowed);
+    return allow_lds(la_sweep_pipe_kernel<T, DKP, NF, NH, REVERSE, DECAY, DENSE, SILU>, lds, lds_allowed);
 }
 
-template <typename T, int DKP, int NF, int NH, bool REVERSE, bool DECAY, bool DENSE>
+template <typename T, int DKP, int NF, int NH, bool REVERSE, bool DECAY, bool DENSE, bool SILU = false>
 static int launch_one(const SweepPair& pair, hipStream_t st) {
     const SweepArgs& a = pair.a[0];
     constexpr size_t lds = PipeLds<DKP, NF, NH>::bytes(sizeof(T));
-    auto kern = la_sweep_pipe_kernel<T, DKP, NF, NH, REVERSE, DECAY, DENSE>;
-    if (const int e = prep_one<T, DKP, NF, NH, REVERSE, DECAY, DENSE>()) return e;
+    auto kern = la_sweep_pipe_kernel<T, DKP, NF, NH, REVERSE, DECAY, DENSE, SILU>;
+    if (const int e = prep_one<T, DKP, NF, NH, REVERSE, DECAY, DENSE, SILU>()) return e;
+    if (SILU != (pair.silu != 0)) return LA_E_UNSUPPORTED;
     const int units8 = (a.bh + 7) / 8 * 8;
     // the slice width the host chose must be one this instantiation's LDS slot and state waves hold
     if (a.zw <= 0 || a.zw > 64 * NH || a.zw % (16 * NH)) return LA_E_UNSUPPORTED;

@@ -7,13 +7,14 @@ outputs are handed to the operator as strided ``(b, h, n, d)`` views and its out
 token-major, so neither the head split before the operator nor the head merge after it copies
 anything (the reference's two ``rearrange`` calls, :56-64, each end in a copy kernel), and the
 output LayerNorm, the sigmoid of the gate and their product (:66-69) are one fused row kernel
-(``lightning_attn.ops.hip.norm_gate``) where the embedding width allows it.
+(``lightning_attn.ops.hip.norm_gate``) where the embedding width allows it.  In inference (no gradient
+wanted) the SiLU on q, k, v (:51-54) runs inside the forward kernel's tile load (``lightning_attn_silu_func``).
 """
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from lightning_attn.ops import lightning_attn_func
+from lightning_attn.ops import lightning_attn_func, lightning_attn_silu_func
 from lightning_attn.ops.hip import norm_gate, norm_gate_supported
 from lightning_attn.utils import _build_slope_tensor
 
@@ -37,14 +38,19 @@ class TnlAttention(nn.Module):
         depth_scale = 1 - layer_idx / (num_layers - 1) + 1e-5
         self.register_buffer("slope_rate", _build_slope_tensor(num_heads) * depth_scale, persistent=False)
         self.fused_norm_gate = True  # False: LayerNorm, sigmoid and product as separate PyTorch operators
+        self.fused_silu = True       # False: SiLU on q, k, v as separate PyTorch operators also without gradients
 
     def _heads(self, t):
         """(b, n, h*d) -> (b, h, n, d) as a view."""
         return t.unflatten(-1, (self.num_heads, self.head_dim)).transpose(-3, -2)
 
     def forward(self, x, **kwargs):
-        q, k, v = (self._heads(F.silu(proj(x))) for proj in (self.q_proj, self.k_proj, self.v_proj))
-        mixed = lightning_attn_func(q, k, v, self.slope_rate)  # (b, h, n, d), token-major memory
+        # SiLU on the projections and the operator (tnl_attn.py:51-56); one kernel when no gradient is wanted
+        q, k, v = (self._heads(proj(x)) for proj in (self.q_proj, self.k_proj, self.v_proj))
+        if self.fused_silu:
+            mixed = lightning_attn_silu_func(q, k, v, self.slope_rate)  # (b, h, n, d), token-major memory
+        else:
+            mixed = lightning_attn_func(F.silu(q), F.silu(k), F.silu(v), self.slope_rate)
         mixed = mixed.transpose(-3, -2).flatten(-2)            # (b, n, h*d): a view of that memory
         gate = self.output_gate(x)
         if self._can_fuse(mixed, gate):

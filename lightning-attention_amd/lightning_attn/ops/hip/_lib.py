@@ -18,7 +18,7 @@ _DTYPES = {torch.bfloat16: LA_BF16, torch.float16: LA_FP16, torch.float32: LA_FP
 SYMBOLS = (
     "la_init", "la_version", "la_error_string", "la_supported", "la_workspace_bytes",
     "la_fwd", "la_bwd", "la_fwd_strided", "la_bwd_strided", "la_workspace_bytes_opts", "la_fwd_opts", "la_bwd_opts",
-    "la_fwd_static", "la_saved_state_bytes", "la_saved_state_interval", "la_fwd_save", "la_bwd_saved",
+    "la_fwd_static", "la_fwd_silu", "la_fwd_silu_supported", "la_saved_state_bytes", "la_saved_state_interval", "la_fwd_save", "la_bwd_saved",
     "srmsnorm_fwd", "srmsnorm_bwd", "norm_gate_supported", "norm_gate_workspace_bytes", "norm_gate_fwd", "norm_gate_bwd",
 )
 
@@ -118,6 +118,10 @@ def lib():
             L.la_bwd_saved.restype = _int
             L.la_bwd_saved.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
                                        _vp, _sz, _op, _vp, _sz, _vp]
+            L.la_fwd_silu_supported.restype = _int
+            L.la_fwd_silu_supported.argtypes = [_i64, _i64, _int]
+            L.la_fwd_silu.restype = _int
+            L.la_fwd_silu.argtypes = L.la_fwd_opts.argtypes
             L.la_fwd_static.restype = _int
             L.la_fwd_static.argtypes = [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp]
             L.srmsnorm_fwd.restype = _int

@@ -61,9 +61,10 @@ def _strides(*tensors):
     return (ctypes.c_int64 * len(vals))(*vals)
 
 
-def _fwd(q, k, v, s, for_backward=False):
+def _fwd(q, k, v, s, for_backward=False, silu=False):
     """Runs the forward pass; returns o, the tensors as the kernels used them and - `for_backward`, where the
-    library has a use for them - the states the backward pass starts its dQ chunks from (else None)."""
+    library has a use for them - the states the backward pass starts its dQ chunks from (else None).
+    `silu`: q, k, v are pre-activations, the kernel applies SiLU as it loads them (forward only)."""
     _lib.require_same_device("lightning_attn2", q=q, k=k, v=v)
     if not (q.dtype == k.dtype == v.dtype):
         raise TypeError("q, k, v must share a dtype")
@@ -87,11 +88,17 @@ def _fwd(q, k, v, s, for_backward=False):
         sp = s.data_ptr() if s is not None else None
         wp = ws.data_ptr() if ws is not None else None
         strides = None if all(t.is_contiguous() for t in (q, k, v, o)) else _strides(q, k, v, o)
-        sv_bytes = _lib.saved_state_bytes(b, h, n, d, e, code, opts) if for_backward else 0
-        saved = torch.empty(sv_bytes // 4, dtype=torch.float32, device=q.device) if sv_bytes else None
-        rc = L.la_fwd_save(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, o.data_ptr(), strides, b, h, n, d, e, code,
-                           wp, ws_bytes, ctypes.byref(opts) if opts is not None else None,
-                           saved.data_ptr() if saved is not None else None, sv_bytes, _lib.stream_ptr(q.device))
+        op = ctypes.byref(opts) if opts is not None else None
+        if silu:
+            saved = None
+            rc = L.la_fwd_silu(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, o.data_ptr(), strides, b, h, n, d, e, code,
+                               wp, ws_bytes, op, _lib.stream_ptr(q.device))
+        else:
+            sv_bytes = _lib.saved_state_bytes(b, h, n, d, e, code, opts) if for_backward else 0
+            saved = torch.empty(sv_bytes // 4, dtype=torch.float32, device=q.device) if sv_bytes else None
+            rc = L.la_fwd_save(q.data_ptr(), k.data_ptr(), v.data_ptr(), sp, o.data_ptr(), strides, b, h, n, d, e, code,
+                               wp, ws_bytes, op, saved.data_ptr() if saved is not None else None, sv_bytes,
+                               _lib.stream_ptr(q.device))
     _lib.check(rc, "la_fwd")
     return o, q, k, v, s, saved
 
@@ -164,3 +171,21 @@ lightning_attn2_no_decay = LightningAttention2NoDecay.apply
 # the chunk-parallel variant of the reference (lightning_attn2_parallel.py:835-1072)
 # computes the same function; the sweep kernels serve it as well
 lightning_attn2_parallel = LightningAttention2.apply
+
+
+def silu_fused_ok(q, k, v):
+    """True when lightning_attn_silu can run as one kernel: HIP tensors of one 16-bit dtype with feature dims
+    the fused forward takes, and no gradient wanted (there is no fused backward pass)."""
+    if not (q.is_cuda and q.dtype in (torch.bfloat16, torch.float16) and q.dtype == k.dtype == v.dtype):
+        return False
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+        return False
+    return bool(_lib.lib().la_fwd_silu_supported(q.shape[-1], v.shape[-1], _lib.dtype_code(q.dtype)))
+
+
+def lightning_attn_silu(q, k, v, s):
+    """lightning_attn2(silu(q), silu(k), silu(v), s) (s None: no decay) as ONE forward kernel, the activation
+    applied where the tiles are loaded: the forward pass of the attention block (examples/module/tnl_attn.py:51-56)
+    without its three activation passes.  Only where silu_fused_ok(q, k, v); not differentiable."""
+    with torch.no_grad():
+        return _fwd(q, k, v, s, False, True)[0]

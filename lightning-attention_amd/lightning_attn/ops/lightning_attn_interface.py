@@ -8,7 +8,7 @@ dims are split into slices of q/k whose partial outputs add up (the scores are
 additive over feature slices) and into column groups of v."""
 import torch
 
-from .hip.lightning_attn2 import lightning_attn2, lightning_attn2_no_decay
+from .hip.lightning_attn2 import lightning_attn2, lightning_attn2_no_decay, lightning_attn_silu, silu_fused_ok
 
 _VARIANTS = ("chunk_loop", "parallel")
 
@@ -59,3 +59,17 @@ def lightning_attn_func(q, k, v, s=None, variant="chunk_loop"):
             o = part if o is None else o + part
         return o
     return run(q, k, v)
+
+
+def lightning_attn_silu_func(q, k, v, s=None, variant="chunk_loop"):
+    """lightning_attn_func(silu(q), silu(k), silu(v), s): what the reference's attention block computes from its
+    projections (examples/module/tnl_attn.py:51-56).  Without a gradient to compute (inference), bf16 / fp16 and
+    feature dims that are multiples of 8 up to 128, the activation is applied inside the forward kernel and the
+    three activation passes disappear; otherwise this is the three PyTorch calls followed by lightning_attn_func."""
+    if variant not in _VARIANTS:
+        raise ValueError("variant must be one of %s, got %r" % (_VARIANTS, variant))
+    d, e = q.shape[-1], v.shape[-1]
+    if d % 8 == 0 and e % 8 == 0 and silu_fused_ok(q, k, v):
+        return lightning_attn_silu(q, k, v, s)
+    f = torch.nn.functional.silu
+    return lightning_attn_func(f(q), f(k), f(v), s, variant)
