@@ -17,6 +17,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build", "obj")
 OUT_DIR = os.path.join(HERE, "lightning_attn", "_C")
 OUT = os.path.join(OUT_DIR, "liblightning_attn_hip.so")
+OUT_TORCH = os.path.join(OUT_DIR, "liblightning_attn_torch.so")
 SOURCES = ["la_api.hip", "la_sweep.hip", "la_sweep_pipe.hip", "la_sweep_pipe_split.hip", "la_sweep_f32.hip", "srmsnorm.hip", "norm_gate.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
@@ -42,7 +43,26 @@ def _compile(src):
     return obj
 
 
-def build(jobs=4, verbose=True):
+def _build_torch_binding():
+    """liblightning_attn_torch.so: the operators as C++ autograd functions over the C ABI (csrc/torch_binding.cpp).
+    Host code only (no device code, no hipify): g++ against PyTorch's headers, linked to the kernel library."""
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = ["g++", "-O2", "-fPIC", "-shared", "-std=c++17", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI), "-Wno-deprecated-declarations"]
+    for inc in ce.include_paths() + ["/opt/rocm/include", os.path.join(ROOT, "include")]:
+        cmd += ["-isystem" if "torch" in inc or "rocm" in inc else "-I", inc]
+    cmd += [os.path.join(CSRC, "torch_binding.cpp"), "-L", tlib, "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch",
+            "-L", OUT_DIR, "-llightning_attn_hip", "-Wl,-rpath,$ORIGIN", "-o", OUT_TORCH]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("torch binding failed to build:\n" + r.stdout + r.stderr)
+    return OUT_TORCH
+
+
+def build(jobs=4, verbose=True, torch_binding=True):
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(OUT_DIR, exist_ok=True)
     with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
@@ -53,10 +73,16 @@ def build(jobs=4, verbose=True):
         raise RuntimeError("link failed:\n" + r.stdout + r.stderr)
     if verbose:
         print("built", OUT)
+    if torch_binding:
+        _build_torch_binding()
+        if verbose:
+            print("built", OUT_TORCH)
     return OUT
 
 
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=4)
-    build(ap.parse_args().jobs)
+    ap.add_argument("--no-torch-binding", action="store_true", help="kernel library only")
+    a = ap.parse_args()
+    build(a.jobs, torch_binding=not a.no_torch_binding)

@@ -22,8 +22,12 @@ SYMBOLS = (
     "srmsnorm_fwd", "srmsnorm_bwd", "norm_gate_supported", "norm_gate_workspace_bytes", "norm_gate_fwd", "norm_gate_bwd",
 )
 
+TORCH_LIB_PATH = os.path.join(_PKG, "_C", "liblightning_attn_torch.so")
+
 _lib = None
-_lock = threading.Lock()
+_lock = threading.RLock()
+_native = None          # torch.ops.lightning_attn_hip, False when the binding is absent or switched off
+_native_enabled = True
 
 _vp, _i64, _int, _sz, _f = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t, ctypes.c_float
 
@@ -138,6 +142,37 @@ def lib():
             L.norm_gate_bwd.argtypes = [_vp] * 11 + [_vp, _sz, _i64, _i64, _int, _vp]
             _lib = L
     return _lib
+
+
+def native_ops():
+    """torch.ops.lightning_attn_hip - the operators as C++ autograd functions over the same C ABI
+    (csrc/torch_binding.cpp), which cost the host a fraction of what the Python autograd nodes do - or None
+    when that library is not built or has been switched off; the Python operators then do the work themselves."""
+    global _native
+    if not _native_enabled:
+        return None
+    if _native is None:
+        with _lock:
+            if _native is None:
+                ops = False
+                if os.path.exists(TORCH_LIB_PATH) and os.path.exists(LIB_PATH):
+                    try:
+                        lib()  # the kernel library first: the binding links against it
+                        torch.ops.load_library(TORCH_LIB_PATH)
+                        ops = torch.ops.lightning_attn_hip
+                        ops.attn, ops.srmsnorm  # resolve now
+                    except (OSError, RuntimeError, AttributeError):
+                        ops = False
+                _native = ops
+    return _native or None
+
+
+def use_native_ops(on):
+    """Switches the C++ autograd path on or off for this process (tests compare the two paths); returns the
+    previous setting."""
+    global _native_enabled
+    prev, _native_enabled = _native_enabled, bool(on)
+    return prev
 
 
 def dtype_code(dtype):

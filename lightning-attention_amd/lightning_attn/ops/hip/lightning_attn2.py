@@ -166,11 +166,42 @@ class LightningAttention2NoDecay(torch.autograd.Function):
         return _bwd(q, k, v, None, do, ctx.la_opts, saved)
 
 
-lightning_attn2 = LightningAttention2.apply
-lightning_attn2_no_decay = LightningAttention2NoDecay.apply
+def _native_ok(q, k, v, s):
+    """Arguments the C++ autograd path takes as they are; anything else goes through the Python operators,
+    which convert what can be converted and raise the documented errors."""
+    if not (q.is_cuda and k.is_cuda and v.is_cuda and q.dtype in _lib._DTYPES and q.dtype == k.dtype == v.dtype):
+        return False
+    if q.dim() != 4 or v.dim() != 4 or k.shape != q.shape or v.shape[:3] != q.shape[:3] or k.device != q.device or v.device != q.device:
+        return False
+    return s is None or (torch.is_tensor(s) and s.numel() == q.shape[1])
+
+
+def _run(q, k, v, s, function):
+    ops = _lib.native_ops()
+    if ops is not None and _native_ok(q, k, v, s):
+        o = _lib.current_opts()
+        if o is None:
+            return ops.attn(q, k, v, s, 0, 0, 0, 0, 0, True)
+        return ops.attn(q, k, v, s, o.chunks, o.scan, o.wide, o.paired, o.once, getattr(o, "save_states", True))
+    return function.apply(q, k, v, s) if function is LightningAttention2 else function.apply(q, k, v)
+
+
+def lightning_attn2(q, k, v, s):
+    """Decayed lightning attention (lightning_attn2.py:398-507): q, k (b,h,n,d), v (b,h,n,e), s h float32 rates.
+    Runs LightningAttention2, as a C++ autograd node where that library is built."""
+    if s is None:
+        raise ValueError("lightning_attn2 needs decay rates s; use lightning_attn2_no_decay")
+    return _run(q, k, v, s, LightningAttention2)
+
+
+def lightning_attn2_no_decay(q, k, v):
+    """lam = 1 variant (lightning_attn2_no_decay.py:367-471)."""
+    return _run(q, k, v, None, LightningAttention2NoDecay)
+
+
 # the chunk-parallel variant of the reference (lightning_attn2_parallel.py:835-1072)
 # computes the same function; the sweep kernels serve it as well
-lightning_attn2_parallel = LightningAttention2.apply
+lightning_attn2_parallel = lightning_attn2
 
 
 def silu_fused_ok(q, k, v):

@@ -132,20 +132,32 @@ def test_saved_states_through_autograd_and_the_opt_out():
     assert _lib.lib().la_saved_state_bytes(b, h, n, d, e, 0, None) > 0
     q, k, v, do = _inputs(b, h, n, d, e, torch.bfloat16, 5)
     s = _build_slope_tensor(h).to(DEV)
-    res = []
-    for save in (True, False):
-        qg, kg, vg = (t.clone().requires_grad_() for t in (q, k, v))
-        with launch_opts(save_states=save):
-            o = lightning_attn_func(qg, kg, vg, s)
-            node_saved = [t for t in o.grad_fn.saved_tensors if t is not None and t.dtype == torch.float32 and t.dim() == 1
-                          and t.numel() > h]
-            assert bool(node_saved) == save
-            o.backward(do)
-        res.append((o.detach(), qg.grad, kg.grad, vg.grad))
-    torch.cuda.synchronize()
-    (o1, dq1, dk1, dv1), (o0, dq0, dk0, dv0) = res
-    assert torch.equal(o1, o0) and torch.equal(dk1, dk0) and torch.equal(dv1, dv0)
-    assert rel_norm(dq1, dq0.float()) < 3e-3
+    per_path = []
+    for native in (True, False):  # the C++ autograd nodes (where built), then the Python ones
+        prev = _lib.use_native_ops(native)
+        try:
+            res = []
+            for save in (True, False):
+                qg, kg, vg = (t.clone().requires_grad_() for t in (q, k, v))
+                with launch_opts(save_states=save):
+                    o = lightning_attn_func(qg, kg, vg, s)
+                    if hasattr(o.grad_fn, "saved_tensors"):  # (Python node)
+                        node_saved = [t for t in o.grad_fn.saved_tensors if t is not None and t.dtype == torch.float32
+                                      and t.dim() == 1 and t.numel() > h]
+                        assert bool(node_saved) == save
+                    o.backward(do)
+                res.append((o.detach(), qg.grad, kg.grad, vg.grad))
+        finally:
+            _lib.use_native_ops(prev)
+        torch.cuda.synchronize()
+        (o1, dq1, dk1, dv1), (o0, dq0, dk0, dv0) = res
+        assert torch.equal(o1, o0) and torch.equal(dk1, dk0) and torch.equal(dv1, dv0)
+        assert rel_norm(dq1, dq0.float()) < 3e-3
+        assert not torch.equal(dq1, dq0)  # the two dQ paths round differently: the states were really used
+        per_path.append(res)
+    for a, c in zip(per_path[0][0] + per_path[0][1], per_path[1][0] + per_path[1][1]):
+        assert torch.equal(a, c)
+    o1 = per_path[0][0][0]
     # no gradient wanted: nothing is saved
     with torch.no_grad():
         o = lightning_attn_func(q, k, v, s)

@@ -226,7 +226,7 @@ def test_triton_import_path_is_an_alias_of_the_hip_operators():
     assert LightningAttention2 is hip.LightningAttention2
     for f in (a1, a2, a3, b1, b2, b3):
         assert callable(f)
-    assert a1.__self__ is hip.LightningAttention2 and a2.__self__ is hip.LightningAttention2NoDecay
+    assert a1 is hip.lightning_attn2 and a2 is hip.lightning_attn2_no_decay and a3 is hip.lightning_attn2_parallel
 
 
 def test_triton_package_names_stay_operators_after_submodule_imports():
