@@ -13,6 +13,9 @@
 //       lightning_attn2_no_decay.py:367-471)
 //   lightning_attn_hip::srmsnorm(x, eps) -> y
 //       _SrmsNorm (lightning_attn/ops/triton/srmsnorm.py:76-175)
+//   lightning_attn_hip::attn_silu(q, k, v, s?, chunks, scan, wide, paired, once) -> o      (no backward pass)
+//   lightning_attn_hip::norm_gate(o, g, weight, bias, eps) -> y
+//       the attention block's activation and gated output norm (examples/module/tnl_attn.py:51-54, 66-69)
 #include <ATen/ATen.h>
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
@@ -210,9 +213,96 @@ struct SrmsNorm : public torch::autograd::Function<SrmsNorm> {
 
 Tensor srmsnorm(const Tensor& x, double eps) { return SrmsNorm::apply(x, eps); }
 
+// attention over silu(q), silu(k), silu(v) in one forward kernel; no backward pass (callers check that none is wanted)
+Tensor attn_silu(const Tensor& q_in, const Tensor& k_in, const Tensor& v_in, const c10::optional<Tensor>& s_in, int64_t chunks,
+                 int64_t scan, int64_t wide, int64_t paired, int64_t once) {
+    const Opts op = make_opts(chunks, scan, wide, paired, once, false);
+    const Tensor q = usable(q_in.detach()), k = usable(k_in.detach()), v = usable(v_in.detach());
+    const int64_t b = q.size(0), h = q.size(1), n = q.size(2), d = q.size(3), e = v.size(3);
+    Tensor s;
+    if (s_in.has_value() && s_in->defined()) {
+        s = s_in->detach();
+        if (s.scalar_type() != at::kFloat || s.device() != q.device() || !s.is_contiguous())
+            s = s.to(q.device(), at::kFloat).contiguous();
+    }
+    const int code = dtype_code(q.scalar_type());
+    const la_launch_opts* lo = op.given ? &op.o : nullptr;
+    Tensor o = at::empty_like(v);
+    const c10::DeviceGuard guard(q.device());
+    const size_t ws_bytes = la_workspace_bytes_opts(0, b, h, n, d, e, code, lo);
+    Tensor ws;
+    if (ws_bytes) ws = at::empty({(int64_t)ws_bytes}, q.options().dtype(at::kByte));
+    int64_t st[4], strides[12];
+    const bool dense = q.is_contiguous() && k.is_contiguous() && v.is_contiguous() && o.is_contiguous();
+    if (!dense) {
+        const Tensor* ts[4] = {&q, &k, &v, &o};
+        for (int i = 0; i < 4; ++i) {
+            norm_strides(*ts[i], st);
+            for (int j = 0; j < 3; ++j) strides[3 * i + j] = st[j];
+        }
+    }
+    check(la_fwd_silu(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.defined() ? s.data_ptr<float>() : nullptr, o.data_ptr(),
+                      dense ? nullptr : strides, b, h, n, d, e, code, ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, lo, stream_of(q)),
+          "la_fwd_silu");
+    return o;
+}
+
+// row-major and 16-byte aligned (a dense view into a larger buffer may start off that grid)
+Tensor dense_rows(const Tensor& t) {
+    const Tensor c = t.is_contiguous() ? t : t.contiguous();
+    return reinterpret_cast<uintptr_t>(c.data_ptr()) % 16 == 0 ? c : c.clone();
+}
+
+// layer_norm(o; weight, bias, eps) * sigmoid(g) over the last dim (examples/module/tnl_attn.py:66-69 of the reference)
+struct NormGate : public torch::autograd::Function<NormGate> {
+    static Tensor forward(AutogradContext* ctx, const Tensor& o, const Tensor& g, const Tensor& weight_in, const Tensor& bias_in,
+                          double eps) {
+        const int64_t cols = o.size(-1);
+        const Tensor o2 = dense_rows(o.reshape({-1, cols})), g2 = dense_rows(g.reshape({-1, cols}));
+        const Tensor weight = dense_rows(weight_in), bias = dense_rows(bias_in);
+        const int64_t rows = o2.size(0);
+        Tensor y = at::empty_like(o2);
+        Tensor mean = at::empty({rows}, o.options().dtype(at::kFloat)), rstd = at::empty({rows}, o.options().dtype(at::kFloat));
+        const c10::DeviceGuard guard(o.device());
+        check(norm_gate_fwd(o2.data_ptr(), g2.data_ptr(), weight.data_ptr(), bias.data_ptr(), y.data_ptr(), mean.data_ptr<float>(),
+                            rstd.data_ptr<float>(), rows, cols, (float)eps, dtype_code(o.scalar_type()), stream_of(o)),
+              "norm_gate_fwd");
+        ctx->save_for_backward({o2, g2, weight, bias, mean, rstd});
+        ctx->saved_data["shape"] = o.sizes().vec();
+        return y.reshape(o.sizes());
+    }
+
+    static variable_list backward(AutogradContext* ctx, variable_list grads) {
+        const auto sv = ctx->get_saved_variables();
+        const Tensor &o2 = sv[0], &g2 = sv[1], &weight = sv[2], &bias = sv[3], &mean = sv[4], &rstd = sv[5];
+        const auto shape = ctx->saved_data["shape"].toIntVector();
+        const int64_t rows = o2.size(0), cols = o2.size(1);
+        Tensor dy = grads[0];
+        TORCH_CHECK(dy.defined() && dy.device() == o2.device(), "norm_gate backward: the upstream gradient is not on ", o2.device());
+        if (dy.scalar_type() != o2.scalar_type()) dy = dy.to(o2.scalar_type());
+        const Tensor dy2 = dense_rows(dy.reshape({rows, cols}));
+        const int code = dtype_code(o2.scalar_type());
+        Tensor d_o = at::empty_like(o2), d_g = at::empty_like(g2), dw = at::empty_like(weight), db = at::empty_like(bias);
+        const c10::DeviceGuard guard(o2.device());
+        const size_t ws_bytes = norm_gate_workspace_bytes(rows, cols, code);
+        Tensor ws = at::empty({(int64_t)std::max<size_t>(ws_bytes, 4)}, o2.options().dtype(at::kByte));
+        check(norm_gate_bwd(o2.data_ptr(), g2.data_ptr(), weight.data_ptr(), bias.data_ptr(), mean.data_ptr<float>(),
+                            rstd.data_ptr<float>(), dy2.data_ptr(), d_o.data_ptr(), d_g.data_ptr(), dw.data_ptr(), db.data_ptr(),
+                            ws.data_ptr(), ws_bytes, rows, cols, code, stream_of(o2)),
+              "norm_gate_bwd");
+        return {d_o.reshape(shape), d_g.reshape(shape), dw, db, Tensor()};
+    }
+};
+
+Tensor norm_gate(const Tensor& o, const Tensor& g, const Tensor& weight, const Tensor& bias, double eps) {
+    return NormGate::apply(o, g, weight, bias, eps);
+}
+
 }  // namespace
 
 TORCH_LIBRARY(lightning_attn_hip, m) {
     m.def("attn", &attn);
     m.def("srmsnorm", &srmsnorm);
+    m.def("attn_silu", &attn_silu);
+    m.def("norm_gate", &norm_gate);
 }

@@ -160,7 +160,7 @@ def native_ops():
                         lib()  # the kernel library first: the binding links against it
                         torch.ops.load_library(TORCH_LIB_PATH)
                         ops = torch.ops.lightning_attn_hip
-                        ops.attn, ops.srmsnorm  # resolve now
+                        ops.attn, ops.srmsnorm, ops.attn_silu, ops.norm_gate  # resolve now
                     except (OSError, RuntimeError, AttributeError):
                         ops = False
                 _native = ops

@@ -218,5 +218,11 @@ def lightning_attn_silu(q, k, v, s):
     """lightning_attn2(silu(q), silu(k), silu(v), s) (s None: no decay) as ONE forward kernel, the activation
     applied where the tiles are loaded: the forward pass of the attention block (examples/module/tnl_attn.py:51-56)
     without its three activation passes.  Only where silu_fused_ok(q, k, v); not differentiable."""
+    ops = _lib.native_ops()
+    if ops is not None and _native_ok(q, k, v, s):
+        o = _lib.current_opts()
+        if o is None:
+            return ops.attn_silu(q, k, v, s, 0, 0, 0, 0, 0)
+        return ops.attn_silu(q, k, v, s, o.chunks, o.scan, o.wide, o.paired, o.once)
     with torch.no_grad():
         return _fwd(q, k, v, s, False, True)[0]

@@ -95,4 +95,9 @@ class _NormGate(torch.autograd.Function):
 def norm_gate(o, g, weight, bias, eps=1e-5):
     """layer_norm(o, (C,), weight, bias, eps) * sigmoid(g) over the last dim; differentiable in
     o, g, weight and bias.  HIP tensors only; see norm_gate_supported for the row widths."""
+    ops = _lib.native_ops()
+    if (ops is not None and o.is_cuda and o.dtype in _lib._DTYPES and o.dtype == g.dtype == weight.dtype == bias.dtype
+            and g.shape == o.shape and o.dim() >= 1 and weight.shape == bias.shape == o.shape[-1:]
+            and g.device == o.device and weight.device == o.device and bias.device == o.device):
+        return ops.norm_gate(o, g, weight, bias, eps)  # the same operator as a C++ autograd node
     return _NormGate.apply(o, g, weight, bias, eps)

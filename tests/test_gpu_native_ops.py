@@ -95,3 +95,29 @@ def test_arguments_the_native_path_does_not_take_raise_as_before():
         lightning_attn_func(q, q, q, _build_slope_tensor(4).to(DEV))
     with pytest.raises(RuntimeError, match="64KB"):
         SimpleRMSNorm(40000)(torch.randn(2, 40000, device=DEV).bfloat16())
+
+
+def test_native_norm_gate_and_silu_forward_match_the_python_paths():
+    from lightning_attn.ops import lightning_attn_silu_func
+    from lightning_attn.ops.hip import norm_gate
+
+    g = torch.Generator().manual_seed(8)
+    rows, cols = 300, 1024
+    o, gate, dy = (torch.randn(2, rows // 2, cols, generator=g).bfloat16().to(DEV) for _ in range(3))
+    w = (1 + 0.1 * torch.randn(cols, generator=g)).bfloat16().to(DEV)
+    b = (0.1 * torch.randn(cols, generator=g)).bfloat16().to(DEV)
+
+    def run():
+        leaves = [t.clone().requires_grad_() for t in (o, gate, w, b)]
+        y = norm_gate(*leaves, 1e-5)
+        y.backward(dy)
+        torch.cuda.synchronize()
+        return [y.detach()] + [t.grad for t in leaves]
+
+    native, python = _both_paths(run)
+    for a, c in zip(native, python):
+        assert torch.equal(a, c)
+    q, k, v = (torch.randn(2, 6, 500, 128, generator=g).bfloat16().to(DEV) for _ in range(3))
+    s = _build_slope_tensor(6).to(DEV)
+    a, c = _both_paths(lambda: lightning_attn_silu_func(q, k, v, s))
+    assert torch.equal(a, c) and not a.requires_grad
