@@ -26,8 +26,19 @@ constexpr unsigned kOob = 0x80000000u;
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, unsigned bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
 }
+// Cache policy of a buffer access (the instruction's auxiliary bits on gfx950): kCached = default; kStream = the nt
+// bit, for data that is touched once - it then does not displace what other accesses of the launch will come back to.
+constexpr int kCached = 0, kStream = 2;
 __device__ __forceinline__ u32x4 buf_load16(__amdgpu_buffer_rsrc_t r, unsigned off) {
     return __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+}
+template <int POLICY>
+__device__ __forceinline__ u32x4 buf_load16p(__amdgpu_buffer_rsrc_t r, unsigned off, unsigned soff = 0u) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, off, soff, POLICY);
+}
+template <int POLICY>
+__device__ __forceinline__ void buf_store16p(__amdgpu_buffer_rsrc_t r, unsigned off, unsigned soff, u32x4 v) {
+    __builtin_amdgcn_raw_buffer_store_b128(v, r, off, soff, POLICY);
 }
 __device__ __forceinline__ void buf_store8(__amdgpu_buffer_rsrc_t r, unsigned off, u32x2 v) {
     __builtin_amdgcn_raw_buffer_store_b64(v, r, off, 0, 0);

@@ -89,6 +89,19 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
     // travels one register set behind them.  NF = 2: the z slice travels with the first feature
     // chunk of its block and is published a block ahead.
     constexpr int ZLAG = (NF == 1 && NH == 2) ? 1 : 0;
+    // Cache policy of the global accesses.  Every tile is needed once per workgroup, and the only second readers
+    // are a sibling workgroup that runs beside this one (the other column slice of the head, which reads the same
+    // x and y; the other sweep of a pair, which reads this sweep's y as its z and the other way round).  Measured
+    // at b4 h32 n8192 d128, la_fwd / la_bwd_saved ms: all cached 0.2253 / 0.5229; x, z and the output streamed, y
+    // cached 0.2153 / 0.4803 (a kernel that only streams this access pattern: 5.3 TB/s with cached, 5.9 TB/s with
+    // streamed accesses).  y stays cached because it is the first of the two touches of a tensor a pair shares (the z
+    // slice of a block is fetched one step after its x / y tiles), so the sibling's streamed z read finds it in L2 -
+    // and because with all four streamed every launch measured slower than with none.  At feature dims above 128
+    // the launches are bound by LDS work and the policy made no difference: left cached.
+    constexpr int PX = NF == 1 ? kStream : kCached;
+    constexpr int PY = kCached;
+    constexpr int PZ = NF == 1 ? kStream : kCached;
+    constexpr int PO = NF == 1 ? kStream : kCached;
     extern __shared__ __align__(16) unsigned char smem[];
     // LDS map in bytes: [3][x 64*XS | y 64*XS] tiles, [NZ][64*ZS] z tiles, [2][64*PS] P tiles.
     // All LDS accesses below are written as (per-step base register) + (compile-time
@@ -242,8 +255,8 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
                 const int c = tid + NL * u;
                 const int row = c / CPX, col = FC0 + (c % CPX) * 8;
                 const unsigned off = col < dk ? ((tok0 + row) * (unsigned)dk + col) * (unsigned)sizeof(T) : kOob;
-                xr[u] = buf_load16(xb, need_x ? off : kOob);
-                yr[u] = buf_load16(yb, valid ? off : kOob);
+                xr[u] = buf_load16p<PX>(xb, need_x ? off : kOob);
+                yr[u] = buf_load16p<PY>(yb, valid ? off : kOob);
             }
             if constexpr (HC == 0) {
                 const unsigned tokz = (unsigned)(tz * 64);
@@ -251,7 +264,7 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
                 for (int u = 0; u < ZC; ++u) {
                     const int row = lane_zrow + ZROWS * u;
                     const unsigned off = lane_zcol < colend ? ((tokz + row) * (unsigned)dv + lane_zcol) * (unsigned)sizeof(T) : kOob;
-                    zr[u] = buf_load16(zb, validz ? off : kOob);
+                    zr[u] = buf_load16p<PZ>(zb, validz ? off : kOob);
                 }
             }
             return;
@@ -266,8 +279,8 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
             for (int u = 0; u < XC; ++u) {
                 // a wave-uniform offset must stay inside the buffer: 0 when none of these rows exists
                 const unsigned tk = u * CROWS < rows ? tok0 + u * CROWS : 0u;
-                xr[u] = buf_load16(xb, lane_row < rows_x - u * CROWS ? lane_x : kOob, tk * xts * (unsigned)sizeof(T));
-                yr[u] = buf_load16(yb, lane_row < rows - u * CROWS ? lane_y : kOob, tk * yts * (unsigned)sizeof(T));
+                xr[u] = buf_load16p<PX>(xb, lane_row < rows_x - u * CROWS ? lane_x : kOob, tk * xts * (unsigned)sizeof(T));
+                yr[u] = buf_load16p<PY>(yb, lane_row < rows - u * CROWS ? lane_y : kOob, tk * yts * (unsigned)sizeof(T));
             }
         } else {
 #pragma unroll
@@ -276,8 +289,8 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
                 const int row = c / CPX, col = FC0 + (c % CPX) * 8;
                 const unsigned ox = col < dk ? (row * xts + col) * (unsigned)sizeof(T) : kOob;
                 const unsigned oy = col < dk ? (row * yts + col) * (unsigned)sizeof(T) : kOob;
-                xr[u] = buf_load16(xb, row < rows_x ? ox : kOob, tok0 * xts * (unsigned)sizeof(T));
-                yr[u] = buf_load16(yb, row < rows ? oy : kOob, tok0 * yts * (unsigned)sizeof(T));
+                xr[u] = buf_load16p<PX>(xb, row < rows_x ? ox : kOob, tok0 * xts * (unsigned)sizeof(T));
+                yr[u] = buf_load16p<PY>(yb, row < rows ? oy : kOob, tok0 * yts * (unsigned)sizeof(T));
             }
         }
         if constexpr (HC == 0) {
@@ -286,7 +299,7 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
 #pragma unroll
             for (int u = 0; u < ZC; ++u) {
                 const unsigned tk = u * ZROWS < rowsz ? tokz + u * ZROWS : 0u;
-                zr[u] = buf_load16(zb, lane_zrow < rowsz - u * ZROWS ? lane_z : kOob, tk * zts * (unsigned)sizeof(T));
+                zr[u] = buf_load16p<PZ>(zb, lane_zrow < rowsz - u * ZROWS ? lane_z : kOob, tk * zts * (unsigned)sizeof(T));
             }
         }
     };
@@ -309,12 +322,12 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
                 // rows >= n fall outside the buffer and are dropped by the hardware range check
                 const unsigned tok0 = (unsigned)(t * 64) + u * ZROWS;
                 const unsigned off = lane_zcol < colend ? ((tok0 + lane_zrow) * (unsigned)dv + lane_zcol) * (unsigned)sizeof(T) : kOob;
-                buf_store16(ob, flush ? off : kOob, 0u, o[u]);
+                buf_store16p<PO>(ob, flush ? off : kOob, 0u, o[u]);
             } else {
                 const unsigned tok0 = flush ? (unsigned)(t * 64) : 0u;
                 const int rows = flush ? (int)min(64u, nrows - tok0) : 0;
                 const unsigned tk = u * ZROWS < rows ? tok0 + u * ZROWS : 0u;
-                buf_store16(ob, lane_zrow < rows - u * ZROWS ? lane_o : kOob, tk * ots * (unsigned)sizeof(T), o[u]);
+                buf_store16p<PO>(ob, lane_zrow < rows - u * ZROWS ? lane_o : kOob, tk * ots * (unsigned)sizeof(T), o[u]);
             }
         }
     };
