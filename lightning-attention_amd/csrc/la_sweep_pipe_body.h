@@ -90,15 +90,18 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
     // chunk of its block and is published a block ahead.
     constexpr int ZLAG = (NF == 1 && NH == 2) ? 1 : 0;
     // Cache policy of the global accesses.  Every tile is needed once per workgroup, and the only second readers
-    // are a sibling workgroup that runs beside this one (the other column slice of the head, which reads the same
-    // x and y; the other sweep of a pair, which reads this sweep's y as its z and the other way round).  Measured
-    // at b4 h32 n8192 d128, la_fwd / la_bwd_saved ms: all cached 0.2253 / 0.5229; x, z and the output streamed, y
-    // cached 0.2153 / 0.4803 (a kernel that only streams this access pattern: 5.3 TB/s with cached, 5.9 TB/s with
-    // streamed accesses).  y stays cached because it is the first of the two touches of a tensor a pair shares (the z
-    // slice of a block is fetched one step after its x / y tiles), so the sibling's streamed z read finds it in L2 -
-    // and because with all four streamed every launch measured slower than with none.  At feature dims above 128
-    // the launches are bound by LDS work and the policy made no difference: left cached.
-    constexpr int PX = NF == 1 ? kStream : kCached;
+    // are a sibling workgroup that runs beside this one: the other 64-column slice of the head, which reads the same
+    // x and y, and the other sweep of a pair, which reads this sweep's y as its z and the other way round.  So the
+    // output and the z slice are streamed (nt), and so is x where no slice shares it (128-column workgroups); y stays
+    // cached: it is the first of the two touches of a tensor a pair shares (the z slice of a block is fetched one
+    // step after its x / y tiles), so the sibling's streamed z read finds it in L2 - and with all four streamed
+    // every launch measured slower than with none.  Measured at b4 h32 n8192 d128, ms: la_fwd (64 columns) 0.2253 all
+    // cached, 0.2207 as here, 0.2153 with x streamed as well - at 1.137 instead of 1.077 GB of HBM traffic, the
+    // sibling slice's read of x then missing L2 now and then: not taken; dQ in 128-column workgroups 0.2078 -> 0.178;
+    // dK + dV 0.315 -> 0.310 at 1.643 instead of 1.726 GB.  (A kernel that only streams this access pattern: 5.3 TB/s
+    // with cached, 5.9 TB/s with streamed accesses.)  At feature dims above 128 the launches are bound by LDS work
+    // and the policy made no difference: left cached.
+    constexpr int PX = (NF == 1 && NH == 2) ? kStream : kCached;
     constexpr int PY = kCached;
     constexpr int PZ = NF == 1 ? kStream : kCached;
     constexpr int PO = NF == 1 ? kStream : kCached;
