@@ -85,13 +85,15 @@ size_t la_workspace_bytes(int which, int64_t b, int64_t h, int64_t n, int64_t d,
  * are bit-identical across all settings except `scan` / `chunks` with a workspace (chunk states
  * summed in another order: equal to rounding).
  */
-enum { LA_OPT_AUTO = 0, LA_OPT_OFF = 1, LA_OPT_ON = 2 };
+enum { LA_OPT_AUTO = 0, LA_OPT_OFF = 1, LA_OPT_ON = 2, LA_OPT_ALL = 3 };
 typedef struct la_launch_opts {
     int32_t chunks; /* sequence chunks per (batch, head, column slice): 0 = library's choice, > 0 forced
                        (at most 64 from scanned states, 8 with warm-up blocks, never more than blocks) */
     int32_t scan;   /* start chunks from scanned states in the workspace: LA_OPT_AUTO (where estimated
                        faster and the workspace suffices) / LA_OPT_OFF (warm-up blocks only)            */
-    int32_t wide;   /* 128 instead of 64 output columns per workgroup (d,e <= 128): AUTO / OFF / ON     */
+    int32_t wide;   /* output columns per workgroup: AUTO / OFF (64) / ON (128, or two equal slices) /
+                       LA_OPT_ALL (d and e in 129..192: all columns in a workgroup of four wavefronts;
+                       as AUTO elsewhere)                                                               */
     int32_t paired; /* backward, d == e: dK and dV in one launch: AUTO (yes) / OFF (one after the other) */
     int32_t once;   /* backward, few sequences: every sweep in one launch: AUTO / OFF / ON               */
 } la_launch_opts;

@@ -18,9 +18,9 @@ int sweep2(const SweepIO& io0, const SweepIO& io1, const float* s, int64_t bh, i
 size_t sweep_workspace_bytes(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int dtype, const Opts& opts);
 SavedPlan plan_saved(int64_t bh, int64_t n, int64_t d, int64_t e, int dtype, const Opts& opts);
 int sweep_saving(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
-                 float* save, int save_len, hipStream_t st);
+                 float* save, int save_len, int width, hipStream_t st);
 int sweep_resumed(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
-                  const float* saved, int nchunk, int chunk_len, hipStream_t st);
+                  const float* saved, int nchunk, int chunk_len, int width, hipStream_t st);
 int prepare_srmsnorm();   // srmsnorm.hip
 int prepare_norm_gate();  // norm_gate.hip
 int sweep_f32(const void* x, const void* y, const void* z, void* out, const float* s, int64_t bh, int64_t h,
@@ -74,8 +74,9 @@ static int check_dims(int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int
 
 static int check_opts(const Opts& o) {
     if (o.chunks < 0) return LA_E_SHAPE;
-    for (int v : {o.scan, o.wide, o.paired, o.once})
+    for (int v : {o.scan, o.paired, o.once})
         if (v != LA_OPT_AUTO && v != LA_OPT_OFF && v != LA_OPT_ON) return LA_E_SHAPE;
+    if (o.wide != LA_OPT_AUTO && o.wide != LA_OPT_OFF && o.wide != LA_OPT_ON && o.wide != LA_OPT_ALL) return LA_E_SHAPE;
     return LA_OK;
 }
 static const Opts kAuto = {0, LA_OPT_AUTO, LA_OPT_AUTO, LA_OPT_AUTO, LA_OPT_AUTO};
@@ -118,7 +119,7 @@ static int fwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s
     if (silu) return sweep_silu(io(q, k, v, o), s, b * h, h, n, d, e, dtype, ws.p, ws.bytes, opts, st);
     if (sv.p) {
         const SavedPlan pl = plan_saved(b * h, n, d, e, dtype, opts);
-        if (saved_usable(sv, pl)) return sweep_saving(io(q, k, v, o), s, b * h, h, n, d, e, dtype, sv.p, pl.chunk_len, st);
+        if (saved_usable(sv, pl)) return sweep_saving(io(q, k, v, o), s, b * h, h, n, d, e, dtype, sv.p, pl.chunk_len, pl.fwd_width, st);
     }
     return run(q, k, v, o, s, b * h, h, n, d, e, dtype, false, ws, opts, st);
 }
@@ -157,17 +158,17 @@ static int bwd(const Tensor& q, const Tensor& k, const Tensor& v, const float* s
         if (rc == LA_OK) return run(k, q, dout, dv, s, b * h, h, n, d, e, dtype, true, ws, opts, st);
         if (rc != LA_E_UNSUPPORTED) return rc;
     }
-    const SavedPlan pl = sv.p ? plan_saved(b * h, n, d, e, dtype, opts) : SavedPlan{1, 0, 0};
+    const SavedPlan pl = sv.p ? plan_saved(b * h, n, d, e, dtype, opts) : SavedPlan{1, 0, 0, 0, 0};
     if (saved_usable(sv, pl) && d == e) {
         // dK + dV first: their reverse walk starts at the end of the sequences, where the forward pass has just
         // been (what the last-level cache still holds of k, v, q is read there: -0.8 % per step at b4 h32 n8192
         // d128), and ends at their start, where the first dQ chunk begins
         rc = sweep2(io(v, dout, q, dk), io(k, q, dout, dv), s, b * h, h, n, d, e, dtype, true, ws.p, ws.bytes, opts, st);
         if (rc != LA_OK) return rc;
-        return sweep_resumed(io(dout, v, k, dq), s, b * h, h, n, e, d, dtype, sv.p, pl.nchunk, pl.chunk_len, st);
+        return sweep_resumed(io(dout, v, k, dq), s, b * h, h, n, e, d, dtype, sv.p, pl.nchunk, pl.chunk_len, pl.dq_width, st);
     }
     if (saved_usable(sv, pl))  // the chunks of dQ start from the states the forward pass left
-        rc = sweep_resumed(io(dout, v, k, dq), s, b * h, h, n, e, d, dtype, sv.p, pl.nchunk, pl.chunk_len, st);
+        rc = sweep_resumed(io(dout, v, k, dq), s, b * h, h, n, e, d, dtype, sv.p, pl.nchunk, pl.chunk_len, pl.dq_width, st);
     else
         rc = run(dout, v, k, dq, s, b * h, h, n, e, d, dtype, false, ws, opts, st);
     if (rc != LA_OK) return rc;

@@ -87,25 +87,28 @@ struct ScanPlan {
 // into the state.  Warm-up blocks: with the geometric chunk lengths of choose_chunks the longest
 // workgroup runs the fraction `frac` of a single walk.  Scanned states: a chunk one and a half times,
 // plus two more launches and the scan (16 us measured, and 10 for the host's share).
-static double block_us(int64_t dk, bool wide) {
+// `width` of a workgroup: 0 = 64 columns of z / out, 1 = 128 (96 where there are 192 to share out), 2 = all
+// (129 .. 192) columns in a workgroup of four wavefronts.
+static const double kWholeBlockUs = 4.2;
+static double block_us(int64_t dk, int width) {
     if (dk <= 64) return 1.0;
-    if (dk <= 128) return wide ? 1.75 : 1.4;
-    if (dk <= 192) return wide ? 3.0 : 2.1;
-    return wide ? 4.1 : 2.9;
+    if (dk <= 128) return width ? 1.75 : 1.4;
+    if (dk <= 192) return width == 2 ? kWholeBlockUs : width ? 3.0 : 2.1;
+    return width ? 4.1 : 2.9;
 }
-// Column slices per sequence: 64 columns each, or - wide - 128.
+// Column slices per sequence: 64 columns each, or 128, or one slice.
 static int64_t wide_slices(int64_t dv) { return (dv + 127) / 128; }
-static int64_t slices(int64_t dk, int64_t dv, bool wide) { return wide ? wide_slices(dv) : (dv + 63) / 64; }
+static int64_t slices(int64_t dk, int64_t dv, int width) { return width == 2 ? 1 : width ? wide_slices(dv) : (dv + 63) / 64; }
 static double warm_up_frac(int64_t wgs, int64_t nblk) {
     static const double frac[9] = {1.0, 1.0, 0.77, 0.71, 0.68, 0.67, 0.66, 0.66, 0.66};
     return frac[warm_up_chunks(wgs, nblk)];
 }
-static double warm_up_us(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, bool wide) {
+static double warm_up_us(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int wide) {
     const int64_t nblk = (n + 63) / 64, wgs = (bh + 7) / 8 * 8 * slices(dk, dv, wide) * nprod;
     return warm_up_frac(wgs, nblk) * (double)nblk * block_us(dk, wide);
 }
 
-static ScanPlan plan_scan(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, bool wide, const Opts& opts) {
+static ScanPlan plan_scan(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int wide, const Opts& opts) {
     const ScanPlan none = {1, 0, 0, warm_up_us(bh, n, dk, dv, nprod, wide)};
     ScanPlan pl = none;
     if (opts.scan == LA_OPT_OFF) return none;
@@ -137,7 +140,9 @@ static ScanPlan plan_scan(int64_t bh, int64_t n, int64_t dk, int64_t dv, int npr
 // as there are workgroups enough.  A 128-column workgroup takes about 1.25 times as long as a
 // 64-column one, and there are half as many: compare the rounds of workgroups the chip has to run.
 // `scratch`: bytes of workspace the caller has.  opts.wide overrides the choice.
-static bool wide_columns(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, size_t scratch, const Opts& opts) {
+static bool wide_columns(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, size_t scratch, const Opts& opts_in) {
+    Opts opts = opts_in;
+    if (opts.wide == LA_OPT_ALL) opts.wide = LA_OPT_AUTO;  // (column_width's business)
     if (dk > 128) {
         // Feature dims 129 .. 256: 128-column workgroups where that makes fewer slices.
         // They pay when the 64-column form needs more rounds of workgroups than the chip has CUs for
@@ -165,27 +170,51 @@ static bool wide_columns(int64_t bh, int64_t n, int64_t dk, int64_t dv, int npro
     return (wide + cus - 1) / cus * 5 < (narrow + cus - 1) / cus * 4;
 }
 
+// Feature dims and columns of 129 .. 192: one workgroup of four wavefronts can take all columns of a sequence
+// (la_sweep_pipe_body.h, NH = 3).  It does per block what two 96-column workgroups do in kWholeBlockUs against
+// 3.0 us each, so it is the form wherever the 64-column one does not already give every workgroup a CU of its own:
+// with that few sequences the narrow workgroups and their chunks spread better over the chip.
+// Returns the width code of the launch: 0 / 1 as wide_columns has it, or 2.  opts.wide overrides the choice.
+static int column_width(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, size_t scratch, const Opts& opts) {
+    const int wide = wide_columns(bh, n, dk, dv, nprod, scratch, opts) ? 1 : 0;
+    if (dk <= 128 || dk > 192 || dv <= 128 || dv > 192) return wide;
+    if (opts.wide != LA_OPT_AUTO) return opts.wide == LA_OPT_ALL ? 2 : wide;
+    const int64_t cus = num_cus(), nblk = (n + 63) / 64, units = (bh + 7) / 8 * 8 * nprod;
+    if (units * slices(dk, dv, 0) <= cus) return wide;
+    auto rounds = [&](int64_t wgs) { return (double)((wgs + cus - 1) / cus); };
+    const double now = rounds(units * slices(dk, dv, wide)) * block_us(dk, wide);
+    const double whole = (units * 2 <= cus ? warm_up_frac(units, nblk) : rounds(units)) * block_us(dk, 2);
+    return whole < now ? 2 : wide;
+}
+
+// The column slices of a sweep whose workgroups have width code `width` (make_args leaves 64-column slices).
+static void set_width(SweepArgs& a, int width, int64_t dv) {
+    if (width == 2) {
+        a.nslice = 1;
+        a.zw = 192;
+    } else if (width) {
+        // equal slices, a whole number of 32-column state waves each (192 columns: 96 + 96, not 128 + 64)
+        const int64_t ws = wide_slices(dv);
+        a.nslice = (int)ws;
+        a.zw = (int)(((dv + ws - 1) / ws + 31) / 32 * 32);
+    }
+}
+
 // Workspace the kernels can use for one launch of nprod sweeps (0: none).
 size_t sweep_workspace_bytes(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int dtype, const Opts& opts) {
     if (dtype != LA_BF16 && dtype != LA_FP16) return 0;
-    return plan_scan(bh, n, dk, dv, nprod, wide_columns(bh, n, dk, dv, nprod, (size_t)-1, opts), opts).bytes;
+    return plan_scan(bh, n, dk, dv, nprod, column_width(bh, n, dk, dv, nprod, (size_t)-1, opts), opts).bytes;
 }
 
 static int launch_planned(SweepPair& p, int64_t bh, int64_t n, int64_t dk, int64_t dv, int dtype, bool reverse, void* ws,
                           size_t ws_bytes, const Opts& opts, hipStream_t st) {
     const bool ws_ok = ws && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0;
-    p.wide = wide_columns(bh, n, dk, dv, p.nprod, ws_ok ? ws_bytes : 0, opts) ? 1 : 0;
+    p.wide = column_width(bh, n, dk, dv, p.nprod, ws_ok ? ws_bytes : 0, opts);
     p.mode = kWarmUp;
     p.chunk_len = 0;
     p.state = nullptr;
-    for (int i = 0; i < p.nprod; ++i)
-        if (p.wide) {
-            // equal slices, a whole number of 32-column state waves each (192 columns: 96 + 96, not 128 + 64)
-            const int64_t ws = wide_slices(dv);
-            p.a[i].nslice = (int)ws;
-            p.a[i].zw = (int)(((dv + ws - 1) / ws + 31) / 32 * 32);
-        }
-    const ScanPlan pl = plan_scan(bh, n, dk, dv, p.nprod, p.wide != 0, opts);
+    for (int i = 0; i < p.nprod; ++i) set_width(p.a[i], p.wide, dv);
+    const ScanPlan pl = plan_scan(bh, n, dk, dv, p.nprod, p.wide, opts);
     if (pl.nchunk > 1 && ws_ok && ws_bytes >= pl.bytes) {
         p.mode = kCollect;  // sweep_pipe runs the three launches
         p.chunk_len = pl.chunk_len;
@@ -233,16 +262,21 @@ int sweep_silu(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t
 // would otherwise be needed to give every CU a workgroup (b*h around 128 on a 256-CU chip).
 // nchunk == 1: not for this shape.
 SavedPlan plan_saved(int64_t bh, int64_t n, int64_t d, int64_t e, int dtype, const Opts& opts) {
-    const SavedPlan none = {1, 0, 0};
+    const SavedPlan none = {1, 0, 0, 0, 0};
     if (dtype != LA_BF16 && dtype != LA_FP16) return none;
-    if (d <= 64 || d > 128 || e > 128) return none;
-    if (opts.chunks != 0 || opts.wide == LA_OPT_ON || opts.scan == LA_OPT_ON) return none;
+    // Feature dims up to 128: the forward pass in 64-column workgroups, dQ in 128-column ones.  d and e both in
+    // 129 .. 192: the forward pass in two slices of up to 96 columns, dQ with all its columns in one workgroup.
+    // (The kernel forms that can leave and pick up the states, la_sweep_pipe_body.h.)
+    const bool big = d > 128 && d <= 192 && e > 128 && e <= 192;
+    if (!big && (d <= 64 || d > 128 || e > 128)) return none;
+    if (opts.chunks != 0 || opts.wide == LA_OPT_ON || opts.wide == LA_OPT_ALL || opts.scan == LA_OPT_ON) return none;
     const int64_t nblk = (n + 63) / 64, cus = num_cus(), units8 = (bh + 7) / 8 * 8;
-    // the forward pass as planned: 64-column workgroups, one walk per sequence
-    if (wide_columns(bh, n, d, e, 1, (size_t)-1, opts)) return none;
-    if (plan_scan(bh, n, d, e, 1, false, opts).nchunk > 1) return none;
-    if (warm_up_chunks(units8 * ((e + 63) / 64), nblk) > 1) return none;
-    // dQ: one 128-column workgroup per sequence and chunk
+    const int fwd_width = big ? 1 : 0, dq_width = big ? 2 : 1;
+    // the forward pass as planned: that width, one walk per sequence
+    if (column_width(bh, n, d, e, 1, (size_t)-1, opts) != fwd_width) return none;
+    if (plan_scan(bh, n, d, e, 1, fwd_width, opts).nchunk > 1) return none;
+    if (warm_up_chunks(units8 * slices(d, e, fwd_width), nblk) > 1) return none;
+    // dQ: one workgroup of that width per sequence and chunk
     int64_t c = cus / units8;
     if (c > nblk / 4) c = nblk / 4;
     if (c > 64) c = 64;
@@ -252,25 +286,31 @@ SavedPlan plan_saved(int64_t bh, int64_t n, int64_t d, int64_t e, int dtype, con
     pl.nchunk = (int)((nblk + pl.chunk_len - 1) / pl.chunk_len);
     if (pl.nchunk < 2) return none;
     // against what the dQ sweep would take by its own plan
-    const bool wide = wide_columns(bh, n, e, d, 1, (size_t)-1, opts);
+    const int wide = column_width(bh, n, e, d, 1, (size_t)-1, opts);
     const ScanPlan own = plan_scan(bh, n, e, d, 1, wide, opts);
-    const double own_us = own.nchunk > 1 ? own.us : warm_up_us(bh, n, e, d, 1, wide);
-    if ((double)pl.chunk_len * block_us(e, true) >= own_us) return none;
+    const int64_t own_wgs = units8 * slices(e, d, wide);
+    const double own_us = own.nchunk > 1 ? own.us
+                          : own_wgs * 2 <= cus ? warm_up_us(bh, n, e, d, 1, wide)
+                                               : (double)((own_wgs + cus - 1) / cus) * (double)nblk * block_us(e, wide);
+    if ((double)pl.chunk_len * block_us(e, dq_width) >= own_us) return none;
     pl.bytes = (size_t)bh * (size_t)(pl.nchunk - 1) * (size_t)(d * e) * sizeof(float);
+    pl.fwd_width = fwd_width;
+    pl.dq_width = dq_width;
     return pl;
 }
 
 // The forward sweep as sweep() plans it where plan_saved applies, leaving its state every save_len blocks in `save`.
 int sweep_saving(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
-                 float* save, int save_len, hipStream_t st) {
+                 float* save, int save_len, int width, hipStream_t st) {
     SweepPair p;
     p.nprod = 1;
     p.a[0] = make_args(io, s, bh, h, n, dk, dv);
+    set_width(p.a[0], width, dv);
     p.a[0].nchunk = 1;
     p.a[0].chunk_start[0] = 0;
     for (int j = 1; j < 9; ++j) p.a[0].chunk_start[j] = (int)((n + 63) / 64);
     p.a[1] = p.a[0];
-    p.wide = 0;
+    p.wide = width;
     p.mode = kWarmUp;
     p.chunk_len = 0;
     p.state = nullptr;
@@ -282,17 +322,16 @@ int sweep_saving(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64
 // The sweep (x, y, z) -> out in nchunk chunks of chunk_len blocks that start from `saved`: what sweep_saving over
 // (., z, y) left behind (per sequence nchunk - 1 row-major dv x dk matrices).  128-column workgroups.
 int sweep_resumed(const SweepIO& io, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk, int64_t dv, int dtype,
-                  const float* saved, int nchunk, int chunk_len, hipStream_t st) {
-    if (dk > 128 || dv > 128 || nchunk < 2 || chunk_len < 1) return LA_E_UNSUPPORTED;
+                  const float* saved, int nchunk, int chunk_len, int width, hipStream_t st) {
+    if (nchunk < 2 || chunk_len < 1 || slices(dk, dv, width) != 1) return LA_E_UNSUPPORTED;
     SweepPair p;
     p.nprod = 1;
     p.a[0] = make_args(io, s, bh, h, n, dk, dv);
-    p.a[0].nslice = 1;
-    p.a[0].zw = 128;
+    set_width(p.a[0], width, dv);
     p.a[0].nchunk = nchunk;
     for (int j = 0; j < 9; ++j) p.a[0].chunk_start[j] = 0;
     p.a[1] = p.a[0];
-    p.wide = 1;
+    p.wide = width;
     p.mode = kResume;
     p.chunk_len = chunk_len;
     p.state = const_cast<float*>(saved);
@@ -324,7 +363,7 @@ int sweep_bwd_once(const SweepIO& dq, const SweepIO& dk, const SweepIO& dv, cons
     if (dtype != LA_BF16 && dtype != LA_FP16) return LA_E_UNSUPPORTED;
     const int forced = opts.once == LA_OPT_ON ? 1 : opts.once == LA_OPT_OFF ? -1 : 0;
     if (forced < 0 || opts.paired == LA_OPT_OFF) return LA_E_UNSUPPORTED;
-    if (forced == 0 && opts.wide == LA_OPT_ON) return LA_E_UNSUPPORTED;  // 128-column workgroups asked for
+    if (forced == 0 && (opts.wide == LA_OPT_ON || opts.wide == LA_OPT_ALL)) return LA_E_UNSUPPORTED;  // wider workgroups asked for
     const int64_t cus = num_cus(), nblk = (n + 63) / 64, nslice = (d + 63) / 64;
     const int64_t wgs = (bh + 7) / 8 * 8 * nslice * 3;  // one chunk each
     if (forced == 0) {
@@ -333,7 +372,7 @@ int sweep_bwd_once(const SweepIO& dq, const SweepIO& dk, const SweepIO& dv, cons
         const bool ws_ok = ws && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0;
         double separate = 0.0;
         for (int nprod = 1; nprod <= 2; ++nprod) {
-            const bool wide = wide_columns(bh, n, d, d, nprod, ws_ok ? ws_bytes : 0, opts);
+            const int wide = column_width(bh, n, d, d, nprod, ws_ok ? ws_bytes : 0, opts);
             const ScanPlan pl = plan_scan(bh, n, d, d, nprod, wide, opts);
             separate += pl.nchunk > 1 && ws_ok && ws_bytes >= pl.bytes ? pl.us : warm_up_us(bh, n, d, d, nprod, wide);
         }
@@ -371,13 +410,13 @@ int sweep_fwd_rev_once(const SweepIO& fwd, const SweepIO& rev, const float* s, i
     if (dtype != LA_BF16 && dtype != LA_FP16) return LA_E_UNSUPPORTED;
     const int forced = opts.once == LA_OPT_ON ? 1 : opts.once == LA_OPT_OFF ? -1 : 0;
     if (forced < 0 || opts.paired == LA_OPT_OFF) return LA_E_UNSUPPORTED;
-    if (forced == 0 && opts.wide == LA_OPT_ON) return LA_E_UNSUPPORTED;
+    if (forced == 0 && (opts.wide == LA_OPT_ON || opts.wide == LA_OPT_ALL)) return LA_E_UNSUPPORTED;
     const int64_t cus = num_cus(), nblk = (n + 63) / 64, nslice = (dv + 63) / 64;
     const int64_t wgs = (bh + 7) / 8 * 8 * nslice * 2;
     if (forced == 0) {
         if (wgs > cus) return LA_E_UNSUPPORTED;
         const bool ws_ok = ws && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0;
-        const bool wide = wide_columns(bh, n, dk, dv, 1, ws_ok ? ws_bytes : 0, opts);
+        const int wide = column_width(bh, n, dk, dv, 1, ws_ok ? ws_bytes : 0, opts);
         const ScanPlan pl = plan_scan(bh, n, dk, dv, 1, wide, opts);
         const double separate = 2.0 * (pl.nchunk > 1 && ws_ok && ws_bytes >= pl.bytes ? pl.us : warm_up_us(bh, n, dk, dv, 1, wide));
         if (warm_up_frac(wgs, nblk) * (double)nblk * block_us(dk, false) >= separate) return LA_E_UNSUPPORTED;

@@ -171,6 +171,7 @@ inline int allow_lds(K kern, size_t lds, unsigned char (&done)[kMaxDevices]) {
 struct SavedPlan {
     int nchunk, chunk_len;
     size_t bytes;
+    int fwd_width, dq_width;  // columns per workgroup (width code of SweepPair::wide) of the pass that saves / resumes
 };
 
 // Launches the single-barrier pipelined kernel (feature dim up to 256); defined in la_sweep_pipe.hip.
@@ -186,9 +187,9 @@ int prepare_plans();
 // Floats of one state slot: the feature dim as the kernel pads it (64, 128, 192 or 256) times the 64 or 128
 // columns of a workgroup.  Must agree with the kernels' own SF; the 128-column form pads feature dims up
 // to 64 to 128.
-inline size_t pipe_state_floats(int dk, bool wide) {
+inline size_t pipe_state_floats(int dk, int wide) {
     const int dkp = dk > 192 ? 256 : dk > 128 ? 192 : (dk <= 64 && !wide ? 64 : 128);
-    return (size_t)dkp * (wide ? 128 : 64);
+    return (size_t)dkp * (wide == 2 ? 192 : wide ? 128 : 64);
 }
 // Between a kCollect and a kApply launch: scans the chunks' end states in place (la_sweep_pipe.hip).
 int launch_state_scan(const SweepPair& p, hipStream_t st);

@@ -87,7 +87,7 @@ __global__ __launch_bounds__(256) void la_state_scan_kernel(float* state, const 
 
 int launch_state_scan(const SweepPair& p, hipStream_t st) {
     const SweepArgs& a = p.a[0];
-    const int quartets = (int)(pipe_state_floats(a.dk, p.wide != 0) / 4);
+    const int quartets = (int)(pipe_state_floats(a.dk, p.wide) / 4);
     const int sets_per_unit = p.nprod * a.nslice;
     hipLaunchKernelGGL(la_state_scan_kernel, dim3((unsigned)((quartets + 255) / 256), (unsigned)(a.bh * sets_per_unit)),
                        dim3(256), 0, st, p.state, a.s, a.h, sets_per_unit, a.nchunk, p.chunk_len, quartets);

@@ -23,6 +23,12 @@
 //   - the P tiles: two LDS buffers (one read, one written);
 //   - the output tile of a block, which the state waves write over the z columns they alone read
 //     and which leaves for memory as whole row segments when that z slot is refilled.
+// NH = 3 is a form of its own for feature dims and column counts of 129 .. 192: one workgroup of FOUR wavefronts
+// covers all (up to 192) columns of a sequence, and every wavefront plays both parts - it fetches and publishes
+// a quarter of the tiles, computes its share of the score tile, and owns three 16-column slabs of the state
+// (144 accumulator registers; with one wavefront per SIMD a wavefront has 512 registers).  The x and y tiles
+// are then read from LDS by four wavefronts per 192 columns instead of six (three state waves in each of two
+// 96-column workgroups), and staged and multiplied into a score tile once per sequence instead of twice.
 // With few (batch, head) sequences the walk is cut into chunks, one workgroup each.  A chunk's
 // incoming state comes either from warm-up blocks (the workgroup first walks everything before its
 // chunk with the state update alone) or, given a workspace, from a scan: the same kernel run once in
@@ -55,7 +61,9 @@ struct PipeLds {
     static constexpr int XY = 2 * 64 * XS;       // elements of one x + y buffer
     static constexpr int ZT = 64 * ZS;           // elements of one z buffer
     static constexpr int PT = 64 * PS;           // elements of one P buffer
-    static constexpr size_t bytes(size_t elt) { return (size_t)(3 * XY + NZ * ZT + 2 * PT) * elt; }
+    // three slabs per state wave: the state waves' decay factors live in LDS, not in registers (512 bytes)
+    static constexpr size_t CF = NH > 2 ? 512 : 0;
+    static constexpr size_t bytes(size_t elt) { return (size_t)(3 * XY + NZ * ZT + 2 * PT) * elt + CF; }
 };
 
 // DENSE: all four tensors are plain (b, h, n, d) arrays; their rows then take a shorter addressing path
@@ -76,12 +84,15 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
     // Threads that fetch, publish and write back the tiles: the 256 of the score waves, which have
     // slack; the state waves' serial chain then holds no memory instructions at all.
     constexpr int NL = 256;
+    constexpr bool MERGED = false;
+    constexpr int NT = MERGED ? 256 : 512;   // threads of the workgroup
     constexpr int CPX = DKH / 8;             // 16-byte chunks per row of an x / y chunk tile
     constexpr int XC = 64 * CPX / NL;        // ... per loader thread
     constexpr bool ROWAL = NL % CPX == 0;    // a thread's chunks lie a whole number of rows apart
     constexpr int ZW = 64 * NH;              // columns of z / out per workgroup
     constexpr int CPR = ZW / 8;              // 16-byte chunks per row of the z slice
     constexpr int ZC = 64 * CPR / NL;        // chunks per loader thread for the z slice / the output tile
+    constexpr bool ZAL = NL % CPR == 0;      // ... which lie a whole number of rows apart (not so at 192 columns)
     constexpr int ZROWS = NL / CPR;          // rows between two of them
     constexpr int NZ = L::NZ;
     // NF = 1, NH = 2: there is room for two z slots only, so the z slice of a block is published one
@@ -101,10 +112,11 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
     // dK + dV 0.315 -> 0.310 at 1.643 instead of 1.726 GB.  (A kernel that only streams this access pattern: 5.3 TB/s
     // with cached, 5.9 TB/s with streamed accesses.)  At feature dims above 128 the launches are bound by LDS work
     // and the policy made no difference: left cached.
+    constexpr bool STREAMS = NF == 1 || NH == 3;  // the forms that come near the memory system's limit
     constexpr int PX = (NF == 1 && NH == 2) ? kStream : kCached;
     constexpr int PY = kCached;
-    constexpr int PZ = NF == 1 ? kStream : kCached;
-    constexpr int PO = NF == 1 ? kStream : kCached;
+    constexpr int PZ = STREAMS ? kStream : kCached;
+    constexpr int PO = STREAMS ? kStream : kCached;
     extern __shared__ __align__(16) unsigned char smem[];
     // LDS map in bytes: [3][x 64*XS | y 64*XS] tiles, [NZ][64*ZS] z tiles, [2][64*PS] P tiles.
     // All LDS accesses below are written as (per-step base register) + (compile-time
@@ -114,6 +126,7 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
     constexpr unsigned E = (unsigned)sizeof(T);
     constexpr unsigned XYB = L::XY * E, ZTB = L::ZT * E, PTB = L::PT * E, YOFF = 64 * XS * E;
     constexpr unsigned ZBASE = 3 * XYB, PBASE = ZBASE + NZ * ZTB;
+    constexpr unsigned CFBASE = PBASE + 2 * PTB;  // (NH = 3) float upd[4][16] by lane group g, float out[16][4] by lane row r
     auto opaque = [](unsigned v) {
         asm volatile("" : "+v"(v));
         return v;
@@ -137,7 +150,7 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const bool state_role = wave >= 4;
+    const bool state_role = MERGED || wave >= 4;
     const int w = wave & 3;
     const int lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int64_t n = a.n;
@@ -171,11 +184,13 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
     //   score waves: cf[4 sl + v]  mask * decay of element v of score tile slot sl
     //   state waves: cf[it]        scale of the inter-block term for token i = 16 it + r
     //                cf[4 + 8 ks + u]  scale of token j = 32 ks + 8 g + u in the state update
-    float cf[20];
+    // (four wavefronts: both sets, the score waves' behind the state waves')
+    constexpr int SC = MERGED ? 20 : 0;
+    float cf[20 + SC];
 #pragma unroll
-    for (int i = 0; i < 20; ++i) cf[i] = 1.f;
+    for (int i = 0; i < 20 + SC; ++i) cf[i] = 1.f;
     float lamB = 1.f;
-    if (!state_role) {
+    if (MERGED || !state_role) {
         const int its[3] = {itA, itB, itB}, jts[3] = {jt0, jt1, jt2};
 #pragma unroll
         for (int sl = 0; sl < 3; ++sl)
@@ -183,9 +198,10 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
             for (int v = 0; v < 4; ++v) {
                 const int i = 16 * its[sl] + r, j = 16 * jts[sl] + 4 * g + v;
                 const int diff = REVERSE ? (j - i) : (i - j);
-                cf[4 * sl + v] = diff >= 0 ? (DECAY ? expf(-rate * (float)diff) : 1.f) : 0.f;
+                cf[SC + 4 * sl + v] = diff >= 0 ? (DECAY ? expf(-rate * (float)diff) : 1.f) : 0.f;
             }
-    } else if (DECAY) {
+    }
+    if (state_role && DECAY) {
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
             const int i = 16 * it + r;
@@ -199,6 +215,21 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
                 cf[4 + 8 * ks + u] = expf(-rate * (float)(REVERSE ? j : 64 - j));
             }
         lamB = expf(-rate * 64.f);
+        if constexpr (NH > 2) {
+            // the factors go to LDS (the same for every state wave; read back where they are used, after the barriers
+            // that precede the walk)
+            if (w == 0) {
+                float* const t = reinterpret_cast<float*>(smem + CFBASE);
+                if (r == 0) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) t[16 * g + i] = cf[4 + i];
+                }
+                if (g == 0) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) t[64 + 4 * r + i] = cf[i];
+                }
+            }
+        }
     }
 
     f32x4 st[NH][KT];  // the state; zeroed where the state waves start their walk
@@ -235,6 +266,11 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
     const int lane_row = tid / CPX, lane_col = (tid % CPX) * 8;
     const int lane_zrow = tid / CPR, lane_zcol = col0 + (tid % CPR) * 8;
     const unsigned lane_z = lane_zcol < colend ? (lane_zrow * zts + lane_zcol) * (unsigned)sizeof(T) : kOob;
+    // chunk u of this thread in the z slice / the output tile: row within the block, first column, element offset in
+    // the LDS slot (not ZAL: 24 chunks per row, every chunk with a row and a column of its own)
+    auto z_row = [&](int u) { return ZAL ? lane_zrow + ZROWS * u : (tid + NL * u) / CPR; };
+    auto z_col = [&](int u) { return ZAL ? lane_zcol : col0 + ((tid + NL * u) % CPR) * 8; };
+    auto z_lds = [&](int u) { return (unsigned)(z_row(u) * ZS + (z_col(u) - col0)) * (unsigned)sizeof(T); };
     // Fetches feature chunk HC of block number b of the walk and, with its first chunk, the z slice
     // that travels with it.  Blocks at or beyond it_end, and the x tile of warm-up blocks, are fetched
     // at the out-of-range offset: zeros, no memory traffic, and the loads are issued unconditionally
@@ -265,8 +301,8 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
                 const unsigned tokz = (unsigned)(tz * 64);
 #pragma unroll
                 for (int u = 0; u < ZC; ++u) {
-                    const int row = lane_zrow + ZROWS * u;
-                    const unsigned off = lane_zcol < colend ? ((tokz + row) * (unsigned)dv + lane_zcol) * (unsigned)sizeof(T) : kOob;
+                    const int row = z_row(u), zc = z_col(u);
+                    const unsigned off = zc < colend ? ((tokz + row) * (unsigned)dv + zc) * (unsigned)sizeof(T) : kOob;
                     zr[u] = buf_load16p<PZ>(zb, validz ? off : kOob);
                 }
             }
@@ -301,8 +337,14 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
             const int rowsz = validz ? (int)min(64u, nrows - tokz) : 0;
 #pragma unroll
             for (int u = 0; u < ZC; ++u) {
-                const unsigned tk = u * ZROWS < rowsz ? tokz + u * ZROWS : 0u;
-                zr[u] = buf_load16p<PZ>(zb, lane_zrow < rowsz - u * ZROWS ? lane_z : kOob, tk * zts * (unsigned)sizeof(T));
+                if constexpr (ZAL) {
+                    const unsigned tk = u * ZROWS < rowsz ? tokz + u * ZROWS : 0u;
+                    zr[u] = buf_load16p<PZ>(zb, lane_zrow < rowsz - u * ZROWS ? lane_z : kOob, tk * zts * (unsigned)sizeof(T));
+                } else {
+                    const int row = z_row(u), zc = z_col(u);
+                    const unsigned oz = zc < colend ? (row * zts + zc) * (unsigned)sizeof(T) : kOob;
+                    zr[u] = buf_load16p<PZ>(zb, row < rowsz ? oz : kOob, tokz * zts * (unsigned)sizeof(T));
+                }
             }
         }
     };
@@ -323,9 +365,15 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
         for (int u = 0; u < ZC; ++u) {
             if (DENSE) {
                 // rows >= n fall outside the buffer and are dropped by the hardware range check
-                const unsigned tok0 = (unsigned)(t * 64) + u * ZROWS;
-                const unsigned off = lane_zcol < colend ? ((tok0 + lane_zrow) * (unsigned)dv + lane_zcol) * (unsigned)sizeof(T) : kOob;
+                const int zc = z_col(u);
+                const unsigned off = zc < colend ? (((unsigned)(t * 64) + z_row(u)) * (unsigned)dv + zc) * (unsigned)sizeof(T) : kOob;
                 buf_store16p<PO>(ob, flush ? off : kOob, 0u, o[u]);
+            } else if constexpr (!ZAL) {
+                const unsigned tok0 = flush ? (unsigned)(t * 64) : 0u;
+                const int rows = flush ? (int)min(64u, nrows - tok0) : 0;
+                const int row = z_row(u), zc = z_col(u);
+                const unsigned oo = zc < colend ? (row * ots + zc) * (unsigned)sizeof(T) : kOob;
+                buf_store16p<PO>(ob, row < rows ? oo : kOob, tok0 * ots * (unsigned)sizeof(T), o[u]);
             } else {
                 const unsigned tok0 = flush ? (unsigned)(t * 64) : 0u;
                 const int rows = flush ? (int)min(64u, nrows - tok0) : 0;
@@ -348,11 +396,12 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
             return __builtin_bit_cast(u32x4, t);
         };
         const unsigned xd = opaque(buf * XYB + (ROWAL ? lane_stage_xy : 0u));
-        const unsigned zd = opaque(ZBASE + zslot * ZTB + lane_stage_z);
+        const unsigned zd = opaque(ZBASE + zslot * ZTB + (ZAL ? lane_stage_z : 0u));
+        auto zoff = [&](int u) { return ZAL ? (unsigned)(u * ZROWS * ZS) * E : z_lds(u); };
         u32x4 o[ZC];
         if constexpr (HC == 0) {
 #pragma unroll
-            for (int u = 0; u < ZC; ++u) o[u] = *reinterpret_cast<const u32x4*>(smem + zd + u * ZROWS * ZS * E);
+            for (int u = 0; u < ZC; ++u) o[u] = *reinterpret_cast<const u32x4*>(smem + zd + zoff(u));
         }
 #pragma unroll
         for (int u = 0; u < XC; ++u) {
@@ -370,7 +419,7 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
         if constexpr (HC == 0) {
             store_out(bout, flush, o);
 #pragma unroll
-            for (int u = 0; u < ZC; ++u) *reinterpret_cast<u32x4*>(smem + zd + u * ZROWS * ZS * E) = SILU ? silu16(zr[u]) : zr[u];
+            for (int u = 0; u < ZC; ++u) *reinterpret_cast<u32x4*>(smem + zd + zoff(u)) = SILU ? silu16(zr[u]) : zr[u];
         }
     };
 
@@ -427,23 +476,23 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
             {
                 V4 p;
 #pragma unroll
-                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[0][v] * cf[v]);
+                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[0][v] * cf[SC + v]);
                 *reinterpret_cast<V4*>(smem + opaque(pbase + (16 * itA * PS + 16 * jt0) * E)) = p;
             }
             if (itB >= 0) {
                 V4 p;
 #pragma unroll
-                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[1][v] * cf[4 + v]);
+                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[1][v] * cf[SC + 4 + v]);
                 *reinterpret_cast<V4*>(smem + opaque(pbase + (16 * itB * PS + 16 * jt1) * E)) = p;
 #pragma unroll
-                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[2][v] * cf[8 + v]);
+                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[2][v] * cf[SC + 8 + v]);
                 *reinterpret_cast<V4*>(smem + opaque(pbase + (16 * itB * PS + 16 * jt2) * E)) = p;
             }
         }
     };
 
     // zero both P buffers once: tiles on the masked side of the diagonal are never written
-    for (int c = tid; c < 2 * L::PT / 8; c += 512) reinterpret_cast<uint4*>(smem + PBASE)[c] = make_uint4(0, 0, 0, 0);
+    for (int c = tid; c < 2 * L::PT / 8; c += NT) reinterpret_cast<uint4*>(smem + PBASE)[c] = make_uint4(0, 0, 0, 0);
     // state-wave lane offsets: x fragment halves (row r, columns 4g..), transposed reads of y and
     // of this wave's 16 z columns (row 8g + r/4, columns 4 (r%4)..), P fragments (row r, chunk g)
     const unsigned lane_xq = (r * XS + 4 * g) * E;
@@ -461,32 +510,39 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
         const int64_t nsave = (nblk - 1) / pair.save_len;  // boundaries per unit
         const int64_t j = (it + 1) / pair.save_len - 1;
         const unsigned lr = opaque((unsigned)r), lg = opaque((unsigned)g);
-        const int c = col0 + cbase + (int)lr;
-        float* const dst = pair.save + ((size_t)unit * nsave + j) * ((size_t)dk * dv) + c;
-        if (c < colend) {
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt)
+        for (int h = 0; h < NH; ++h) {
+            const int c = col0 + cbase + 16 * h + (int)lr;
+            float* const dst = pair.save + ((size_t)unit * nsave + j) * ((size_t)dk * dv) + c;
+            if (c < colend) {
 #pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const int k = 16 * kt + 4 * (int)lg + v;
-                    if (k < dk) dst[(size_t)k * dv] = st[0][kt][v];
-                }
+                for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int k = 16 * kt + 4 * (int)lg + v;
+                        if (k < dk) dst[(size_t)k * dv] = st[h][kt][v];
+                    }
+            }
         }
     };
+    // the forms a forward pass that saves runs in, and the forms a pass that resumes runs in
+    constexpr bool SAVES = !REVERSE && ((NH == 1 && NF == 1) || (NH == 2 && NF == 2));
+    constexpr bool RESUMES = !REVERSE && ((NH == 2 && NF == 1) || (NH == 3 && NF == 2));
 
     f32x4 oacc[NH][4];  // state waves: the output tile of the block in progress, summed over the feature chunks
 
     // One step: feature chunk HF of block `it`; step number s = NF it + HF.  `xr, yr, zr` hold step
     // s+2 on entry and step s+4 on exit.
+    // `role`: 0 the score waves' part of the step, 1 the state waves', 2 both (four wavefronts).
     auto iteration = [&](auto role, auto hf, const int64_t it, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4 (&zr)[ZC]) __attribute__((always_inline)) {
-        constexpr bool STATE = decltype(role)::value;
+        constexpr int ROLE = decltype(role)::value;
         constexpr int HF = decltype(hf)::value;
         const bool have_next = it + 1 < it_end;
         const bool warm = it < it_first;  // warm-up block: state update only
         const int bcur = (int)((unsigned)(it * NF + HF) % 3u);
         const int bnext = bcur == 2 ? 0 : bcur + 1;
         const int bstage = bnext == 2 ? 0 : bnext + 1;
-        if constexpr (!STATE) {
+        if constexpr (ROLE != 1) {
             // publish step s+2 (its buffer was last read in step s-1; the z slot that goes with it
             // still holds an output tile) and refill the registers with step s+4
             constexpr int HS = (HF + 2) % NF, HL = (HF + 4) % NF, HC = (HF + 1) % NF;
@@ -497,7 +553,8 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
             // the score tile runs one step ahead of the state waves
             const int64_t bc = it + (HF + 1) / NF;
             if (bc < it_end && bc >= it_first) score_step(std::integral_constant<int, HC>{}, bnext, (int)(bc & 1));
-        } else if (cols_active) {
+        }
+        if (ROLE != 0 && cols_active) {
             const unsigned xq = opaque(bcur * XYB + lane_xq);
             const unsigned yq = opaque(bcur * XYB + YOFF + lane_yt);
             const int zcur = NZ == 3 ? bcur : (int)(it & 1);  // z / out slot of this block
@@ -505,12 +562,18 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
             const unsigned pq = opaque(PBASE + (unsigned)(it & 1) * PTB + lane_pr);
             // z^T fragments of this wave's 16-column slabs: A operand of the intra-block product
             // and, scaled, B operand of the state update
+            // (three slabs: the state takes 144 registers; the fragments are fetched where they are first needed, the
+            // x and P fragments without look-ahead, the y^T fragments two tiles at a time)
+            constexpr bool LEAN = NH > 2;
             V8 zf[NH][2];
+            auto read_z = [&]() {
 #pragma unroll
-            for (int h = 0; h < NH; ++h)
+                for (int h = 0; h < NH; ++h)
 #pragma unroll
-                for (int ks = 0; ks < 2; ++ks)
-                    zf[h][ks] = cat<V8, V4>(ldt(zq + (32 * ks * ZS + 16 * h) * E), ldt(zq + ((32 * ks + 4) * ZS + 16 * h) * E));
+                    for (int ks = 0; ks < 2; ++ks)
+                        zf[h][ks] = cat<V8, V4>(ldt(zq + (32 * ks * ZS + 16 * h) * E), ldt(zq + ((32 * ks + 4) * ZS + 16 * h) * E));
+            };
+            if constexpr (!LEAN) read_z();
             if (!warm) {
                 // out^T[c][i] = Lout[i] * sum_k state[k][c] x[i][k]  +  sum_j z[j][c] P[i][j]
                 // One slab: all x fragments are requested up front; LDS answers in order, so the
@@ -518,9 +581,10 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
                 // the later ones are still on their way.  Two slabs: every fragment feeds both, and
                 // there are registers for one step of look-ahead only.
                 // (256 features and two slabs: the state takes 128 registers, no look-ahead)
-                constexpr int NBX = NH == 1 ? KSH : (NF == 2 && KTH > 6) ? 1 : 2;
+                constexpr int NBX = NH == 1 ? KSH : ((NF == 2 && KTH > 6) || LEAN) ? 1 : 2;
+                constexpr bool XALL = NBX == KSH;
                 V8 bx[NBX][4];
-                V8 bp[4][2];
+                V8 bp[LEAN ? 2 : 4][2];
                 auto read_x = [&](int ks) {
 #pragma unroll
                     for (int i4 = 0; i4 < 4; ++i4) {
@@ -544,7 +608,7 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
                     __builtin_amdgcn_sched_barrier(0);
                 };
 #pragma unroll
-                for (int ks = 0; ks < (NH == 1 ? KSH : NBX - 1); ++ks) read_x(ks);
+                for (int ks = 0; ks < (XALL ? KSH : NBX - 1); ++ks) read_x(ks);
                 if constexpr (HF == 0) {
 #pragma unroll
                     for (int h = 0; h < NH; ++h)
@@ -553,9 +617,23 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
                 }
 #pragma unroll
                 for (int ks = 0; ks < KSH; ++ks) {
-                    if (NH > 1 && NBX == 2 && ks + 1 < KSH) read_x(ks + 1);
-                    if (NH > 1 && NBX == 1) read_x(ks);
+                    if (!XALL && NBX == 2 && ks + 1 < KSH) read_x(ks + 1);
+                    if (!XALL && NBX == 1) read_x(ks);
                     constexpr int KG0 = HF * KSH;  // contraction steps of the chunks before this one
+                    if constexpr (LEAN) {
+                        // slab by slab: one converted state fragment at a time
+#pragma unroll
+                        for (int h = 0; h < NH; ++h) {
+                            V8 sb1;
+#pragma unroll
+                            for (int v = 0; v < 4; ++v) {
+                                sb1[v] = M::cvt(st[h][2 * (KG0 + ks)][v]);
+                                sb1[4 + v] = M::cvt(st[h][2 * (KG0 + ks) + 1][v]);
+                            }
+#pragma unroll
+                            for (int i4 = 0; i4 < 4; ++i4) oacc[h][i4] = M::mma(sb1, bx[ks % NBX][i4], oacc[h][i4]);
+                        }
+                    } else {
                     V8 sb[NH];
 #pragma unroll
                     for (int h = 0; h < NH; ++h)
@@ -569,29 +647,47 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
                     for (int i4 = 0; i4 < 4; ++i4)
 #pragma unroll
                         for (int h = 0; h < NH; ++h) oacc[h][i4] = M::mma(sb[h], bx[ks % NBX][i4], oacc[h][i4]);
+                    }
                     __builtin_amdgcn_sched_barrier(0);
                     // the P fragments follow once half of the x fragments have been used up
-                    if (HF == NF - 1 && NH == 1 && ks == (KSH - 1) / 2) read_p();
+                    if (HF == NF - 1 && XALL && ks == (KSH - 1) / 2) read_p();
                 }
                 if constexpr (HF == NF - 1) {
-                    if (NH > 1) read_p();
+                    if constexpr (LEAN) read_z();
+                    if (!XALL && !LEAN) read_p();
                     if (DECAY) {
+                        f32x4 co;
+                        if constexpr (LEAN) co = *reinterpret_cast<const f32x4*>(smem + opaque(CFBASE + 256 + 16 * r));
 #pragma unroll
                         for (int h = 0; h < NH; ++h)
 #pragma unroll
                             for (int i4 = 0; i4 < 4; ++i4)
 #pragma unroll
-                                for (int v = 0; v < 4; ++v) oacc[h][i4][v] *= cf[i4];
+                                for (int v = 0; v < 4; ++v) oacc[h][i4][v] *= LEAN ? co[i4] : cf[i4];
                     }
 #pragma unroll
                     for (int i4 = 0; i4 < 4; ++i4) {
+                        if constexpr (LEAN) {
+                            // the P fragments of two 16-row tiles at a time
+                            if (i4 % 2 == 0) {
+#pragma unroll
+                                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                                    for (int k2 = 0; k2 < 2; ++k2) {
+                                        const bool need = REVERSE ? (k2 >= (i4 + j) / 2) : (k2 <= (i4 + j) / 2);
+                                        if (need) bp[j][k2] = ld8(pq + (16 * (i4 + j) * PS + 32 * k2) * E);
+                                    }
+                                __builtin_amdgcn_sched_barrier(0);
+                            }
+                        }
 #pragma unroll
                         for (int ks = 0; ks < 2; ++ks) {
                             const bool need = REVERSE ? (ks >= i4 / 2) : (ks <= i4 / 2);
 #pragma unroll
                             for (int h = 0; h < NH; ++h)
-                                if (need) oacc[h][i4] = M::mma(zf[h][ks], bp[i4][ks], oacc[h][i4]);
+                                if (need) oacc[h][i4] = M::mma(zf[h][ks], bp[LEAN ? i4 % 2 : i4][ks], oacc[h][i4]);
                         }
+                        if (LEAN && i4 % 2 == 1) __builtin_amdgcn_sched_barrier(0);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                     // leave the tile in the z slot of this block, over this wave's own z columns (read
@@ -612,7 +708,23 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
                 // state = lam^64 state + y^T (z * Lupd), the rows of this feature chunk
                 constexpr int KT0 = HF * KTH;
                 // transposed y reads in batches where the state leaves no registers for all of them at once
-                constexpr int UB = (NF == 2 && NH == 2 && KTH > 6) ? 4 : KTH;
+                constexpr int UB = (NF == 2 && NH == 2 && KTH > 6) ? 4 : LEAN ? 2 : KTH;
+                if constexpr (LEAN) {
+                    if (HF != NF - 1 || warm) read_z();
+                    if (DECAY) {
+                        // (scaled before the y^T fragments are fetched: the factors and the fragments never share registers)
+#pragma unroll
+                        for (int ks = 0; ks < 2; ++ks) {
+                            const unsigned ca = opaque(CFBASE + (16 * g + 8 * ks) * 4);
+                            const f32x4 c0 = *reinterpret_cast<const f32x4*>(smem + ca), c1 = *reinterpret_cast<const f32x4*>(smem + ca + 16);
+#pragma unroll
+                            for (int h = 0; h < NH; ++h)
+#pragma unroll
+                                for (int u = 0; u < 8; ++u) zf[h][ks][u] = (T)((float)zf[h][ks][u] * (u < 4 ? c0[u] : c1[u - 4]));
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
 #pragma unroll
                 for (int t0 = 0; t0 < KTH; t0 += UB) {
                     V8 ay[UB][2];
@@ -631,7 +743,8 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
 #pragma unroll
                             for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-                                for (int u = 0; u < 8; ++u) zf[h][ks][u] = (T)((float)zf[h][ks][u] * cf[4 + 8 * ks + u]);
+                                for (int u = 0; u < 8; ++u)
+                                    if (!LEAN) zf[h][ks][u] = (T)((float)zf[h][ks][u] * cf[4 + 8 * ks + u]);
 #pragma unroll
                             for (int kt = 0; kt < KTH; ++kt)
 #pragma unroll
@@ -648,7 +761,7 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
-            if constexpr (!REVERSE && NH == 1 && NF == 1) {
+            if constexpr (SAVES && HF == NF - 1) {
                 // a boundary the next pass over these tensors may start from: leave the state after block `it`
                 if (it + 1 == next_save) {
                     save_state(it);
@@ -684,17 +797,17 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
     // the last block's output tile is still in its z slot when the walk ends
     auto flush_last = [&]() {
         if (it_end <= it_first) return;
-        const unsigned zd = ZBASE + (unsigned)(NZ == 3 ? (it_end - 1) % 3 : (it_end - 1) & 1) * ZTB + lane_stage_z;
+        const unsigned zd = ZBASE + (unsigned)(NZ == 3 ? (it_end - 1) % 3 : (it_end - 1) & 1) * ZTB + (ZAL ? lane_stage_z : 0u);
         u32x4 o[ZC];
 #pragma unroll
-        for (int u = 0; u < ZC; ++u) o[u] = *reinterpret_cast<const u32x4*>(smem + zd + u * ZROWS * ZS * E);
+        for (int u = 0; u < ZC; ++u) o[u] = *reinterpret_cast<const u32x4*>(smem + zd + (ZAL ? (unsigned)(u * ZROWS * ZS) * E : z_lds(u)));
         store_out(it_end - 1, true, o);
     };
     // The two kinds of waves part here for good, prologue included (two barriers in each branch):
     // the compiler lays the branches out one after the other and keeps alive, while the first one
     // runs, whatever the second one needs of the values computed before this point - which must
     // therefore not include the score waves' prefetch registers.
-    if (!state_role) {
+    auto prologue = [&]() __attribute__((always_inline)) {
         const int b0 = (int)((unsigned)(it0 * NF) % 3u), b1 = b0 == 2 ? 0 : b0 + 1;
         if constexpr (NF == 1) {
             load_step(C0{}, it0, xrA, yrA, zrA);
@@ -714,14 +827,9 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
         __syncthreads();
         if (it0 >= it_first && it0 < it_end) score_step(C0{}, b0, (int)(it0 & 1));
         __syncthreads();
-        walk(std::false_type{});
-        flush_last();
-    } else {
-        __syncthreads();
-        __syncthreads();
-        // The state waves are the critical path and every SIMD holds one wave of each kind: when both
-        // have an instruction ready (right after the barrier all eight waves go for LDS), theirs goes first.
-        __builtin_amdgcn_s_setprio(1);
+    };
+    // the state a workgroup starts from: zero, or what the scan (kApply) or the pass before (kResume) left
+    auto init_state = [&]() __attribute__((always_inline)) {
         // this lane's part of a state slot: [wave][slab][tile][lane] accumulator quartets
         const size_t lane_slot = ((size_t)w * NH * KT * 64 + lane) * 4;
         const bool resume = mode == kApply && chunk > 0;
@@ -731,7 +839,7 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
                 st[h][kt] = resume ? *reinterpret_cast<const f32x4*>(src + (size_t)(h * KT + kt) * 256) : (f32x4){0.f, 0.f, 0.f, 0.f};
-        if constexpr (!REVERSE && NH == 2 && NF == 1) {
+        if constexpr (RESUMES) {
             if (mode == kResume && chunk > 0) {
                 // state[k][c] = saved[c][k]: this lane's four k of a tile are neighbours in row c of the saved matrix
                 const float* const m = pair.state + ((size_t)unit * (nchunk - 1) + (chunk - 1)) * ((size_t)dk * dv);
@@ -746,14 +854,36 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
                 }
             }
         }
-        walk(std::true_type{});
+    };
+    auto leave_state = [&]() __attribute__((always_inline)) {
         if (mode == kCollect) {
+            const size_t lane_slot = ((size_t)w * NH * KT * 64 + lane) * 4;
             float* const dst = slot0 + (size_t)chunk * SF + lane_slot;
 #pragma unroll
             for (int h = 0; h < NH; ++h)
 #pragma unroll
                 for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<f32x4*>(dst + (size_t)(h * KT + kt) * 256) = st[h][kt];
         }
+    };
+    if constexpr (MERGED) {
+        prologue();
+        init_state();
+        walk(std::integral_constant<int, 2>{});
+        flush_last();
+        leave_state();
+    } else if (!state_role) {
+        prologue();
+        walk(std::integral_constant<int, 0>{});
+        flush_last();
+    } else {
+        __syncthreads();
+        __syncthreads();
+        // The state waves are the critical path and every SIMD holds one wave of each kind: when both
+        // have an instruction ready (right after the barrier all eight waves go for LDS), theirs goes first.
+        __builtin_amdgcn_s_setprio(1);
+        init_state();
+        walk(std::integral_constant<int, 1>{});
+        leave_state();
     }
 }
 
@@ -789,11 +919,14 @@ static int launch_one(const SweepPair& pair, hipStream_t st) {
     // the slice width the host chose must be one this instantiation's LDS slot and state waves hold
     if (a.zw <= 0 || a.zw > 64 * NH || a.zw % (16 * NH)) return LA_E_UNSUPPORTED;
     // the state slots the host sized must be the ones this instantiation reads and writes
-    if ((pair.mode == kCollect || pair.mode == kApply) && pipe_state_floats(a.dk, pair.wide != 0) != (size_t)4 * NH * (DKP / 16) * 64 * 4)
+    if ((pair.mode == kCollect || pair.mode == kApply) && pipe_state_floats(a.dk, pair.wide) != (size_t)4 * NH * (DKP / 16) * 64 * 4)
         return LA_E_WORKSPACE;
+    if (pair.wide != NH - 1) return LA_E_UNSUPPORTED;
     // the plain-matrix forms of the state exist in two instantiations only
-    if (pair.mode == kResume && (REVERSE || NH != 2 || NF != 1 || pair.nprod != 1)) return LA_E_UNSUPPORTED;
-    if (pair.save && (REVERSE || NH != 1 || NF != 1 || pair.nprod != 1 || pair.mode != kWarmUp || a.nchunk != 1)) return LA_E_UNSUPPORTED;
+    constexpr bool SAVES = !REVERSE && ((NH == 1 && NF == 1) || (NH == 2 && NF == 2));
+    constexpr bool RESUMES = !REVERSE && ((NH == 2 && NF == 1) || (NH == 3 && NF == 2));
+    if (pair.mode == kResume && (!RESUMES || pair.nprod != 1)) return LA_E_UNSUPPORTED;
+    if (pair.save && (!SAVES || pair.nprod != 1 || pair.mode != kWarmUp || a.nchunk != 1)) return LA_E_UNSUPPORTED;
     const unsigned grid = (unsigned)(units8 * a.nslice * a.nchunk * pair.nprod);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, st, pair);
     return (int)hipGetLastError();
@@ -836,7 +969,7 @@ static int prep_family() {
     LA_P(false, false, false) LA_P(false, false, true) LA_P(false, true, false) LA_P(false, true, true)
     LA_P(true, false, false) LA_P(true, false, true) LA_P(true, true, false) LA_P(true, true, true)
 #undef LA_P
-    if (NH == 1) {
+    if constexpr (NH == 1) {
 #define LA_P(D, S) if (!e) e = prep_both_one<T, DKP, NF, D, S>();
         LA_P(false, false) LA_P(false, true) LA_P(true, false) LA_P(true, true)
 #undef LA_P

@@ -14,6 +14,7 @@ static int launch_split_dir(const SweepPair& pair, hipStream_t st) {
     const bool dense = all_plain(pair);
 #define LA_GO2(DKP, NH, DENSE) (decay ? launch_one<T, DKP, 2, NH, REVERSE, true, DENSE>(pair, st) : launch_one<T, DKP, 2, NH, REVERSE, false, DENSE>(pair, st))
 #define LA_GO(DKP, NH) (dense ? LA_GO2(DKP, NH, true) : LA_GO2(DKP, NH, false))
+    if (pair.wide == 2) return a.dk <= 192 ? LA_GO(192, 3) : LA_E_UNSUPPORTED;
     if (a.dk <= 192) return pair.wide ? LA_GO(192, 2) : LA_GO(192, 1);
     return pair.wide ? LA_GO(256, 2) : LA_GO(256, 1);
 #undef LA_GO
@@ -51,10 +52,12 @@ int launch_split_both(const SweepBoth& b, int dtype, hipStream_t st) {
 int prepare_split() {
     int e = prep_family<__bf16, 192, 2, 1>();
     if (!e) e = prep_family<__bf16, 192, 2, 2>();
+    if (!e) e = prep_family<__bf16, 192, 2, 3>();
     if (!e) e = prep_family<__bf16, 256, 2, 1>();
     if (!e) e = prep_family<__bf16, 256, 2, 2>();
     if (!e) e = prep_family<_Float16, 192, 2, 1>();
     if (!e) e = prep_family<_Float16, 192, 2, 2>();
+    if (!e) e = prep_family<_Float16, 192, 2, 3>();
     if (!e) e = prep_family<_Float16, 256, 2, 1>();
     if (!e) e = prep_family<_Float16, 256, 2, 2>();
     return e;

@@ -31,7 +31,7 @@ _native_enabled = True
 
 _vp, _i64, _int, _sz, _f = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t, ctypes.c_float
 
-LA_OPT_AUTO, LA_OPT_OFF, LA_OPT_ON = 0, 1, 2
+LA_OPT_AUTO, LA_OPT_OFF, LA_OPT_ON, LA_OPT_ALL = 0, 1, 2, 3
 
 
 class LaunchOpts(ctypes.Structure):
@@ -52,6 +52,8 @@ def current_opts():
 
 
 def _tri(v):
+    if v == "all":  # (wide only) every column of a sequence in one workgroup, LA_OPT_ALL
+        return LA_OPT_ALL
     return LA_OPT_AUTO if v is None else (LA_OPT_ON if v else LA_OPT_OFF)
 
 

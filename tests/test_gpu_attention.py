@@ -568,7 +568,7 @@ def test_feature_dims_off_the_grid_of_8_are_padded(b, h, n, d, e, dtype):
     check(got, want, dtype, "padded dims %s" % ((b, h, n, d, e),))
 
 
-@pytest.mark.parametrize("b, h, n, d, e", [(2, 3, 700, 192, 192), (1, 2, 450, 256, 256), (1, 3, 513, 160, 160), (2, 2, 300, 136, 200),
+@pytest.mark.parametrize("b, h, n, d, e", [(2, 3, 700, 192, 192), (1, 2, 450, 256, 256), (1, 3, 513, 160, 160), (2, 2, 300, 136, 200), (2, 2, 333, 176, 144),
                                            (1, 2, 330, 192, 256), (1, 1, 200, 256, 72), (1, 2, 260, 144, 96), (1, 2, 1000, 224, 232)])
 @pytest.mark.parametrize("decay", [True, False])
 def test_wide_two_barrier_kernel_is_bit_identical_to_the_64_column_form(b, h, n, d, e, decay):
@@ -588,6 +588,16 @@ def test_wide_two_barrier_kernel_is_bit_identical_to_the_64_column_form(b, h, n,
     for name, a, c in zip(("o", "dq", "dk", "dv"), scanned, narrow):
         assert rel_norm(a, c) < 5e-4, name
     check(scanned, want, torch.bfloat16, "wide, scanned chunks %s" % ((b, h, n, d, e),))
+    if 128 < d <= 192 and 128 < e <= 192:
+        # all (up to 192) columns of a sequence in one workgroup, three accumulator slabs per state wave
+        for opts in ({"chunks": 1}, {"chunks": 3}, {"chunks": 2, "paired": False}):
+            whole = run_hip(q, k, v, s, do, wide="all", scan=False, once=False, **opts)
+            for name, a, c in zip(("o", "dq", "dk", "dv"), whole, narrow):
+                assert torch.equal(a, c), ("all columns", opts, name)
+        scanned = run_hip(q, k, v, s, do, wide="all", chunks=4, once=False)
+        for name, a, c in zip(("o", "dq", "dk", "dv"), scanned, narrow):
+            assert rel_norm(a, c) < 5e-4, name
+        check(scanned, want, torch.bfloat16, "all columns, scanned chunks %s" % ((b, h, n, d, e),))
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
