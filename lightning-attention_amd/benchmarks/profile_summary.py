@@ -38,8 +38,8 @@ def classify(name):
              or re.search(r"<[^,]+, *(\d+), *(\d), *(\d), *(true|false|0|1)", name))
         if not m:
             return "sweep_pipe"
-        dkp, rev, wide = int(m.group(1)), m.group(4) in ("1", "true"), m.group(3) == "2"
-        key = ("reverse" if rev else "forward") + ("_pair" if rev and wide else "_wide" if wide else "")
+        dkp, rev, wide, whole = int(m.group(1)), m.group(4) in ("1", "true"), m.group(3) == "2", m.group(3) == "3"
+        key = ("reverse" if rev else "forward") + ("_all" if whole else "_pair" if rev and wide else "_wide" if wide else "")
         return key if dkp <= 128 else "d%d_%s" % (dkp, key)
     if "la_state_scan" in name:
         return "state_scan"
