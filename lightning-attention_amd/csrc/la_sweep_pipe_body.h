@@ -110,12 +110,17 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
     // cached, 0.2207 as here, 0.2153 with x streamed as well - at 1.137 instead of 1.077 GB of HBM traffic, the
     // sibling slice's read of x then missing L2 now and then: not taken; dQ in 128-column workgroups 0.2078 -> 0.178;
     // dK + dV 0.315 -> 0.310 at 1.643 instead of 1.726 GB.  (A kernel that only streams this access pattern: 5.3 TB/s
-    // with cached, 5.9 TB/s with streamed accesses.)  At feature dims above 128 the launches are bound by LDS work
-    // and the policy made no difference: left cached.
+    // with cached, 5.9 TB/s with streamed accesses.)  At feature dims above 128 the launches in 64- and 96- / 128-column
+    // workgroups are bound by LDS work and the policy made no difference: left cached.  With all columns in one
+    // workgroup (NH = 3) they come near the memory side's limit for tiles fetched in half rows (4.6 - 4.8 TB/s for
+    // a kernel that only streams that pattern): there the output is streamed, x and y stay cached (the 128-byte
+    // line in the middle of a 384-byte row belongs to both halves and is asked for twice, half a block apart), and
+    // z is streamed only when walking forward - walking backward the launch is a dK + dV pair, whose z reads are
+    // the sibling sweep's y reads of the same moment (b4 h32 n8192 d192: 2.42 instead of 2.74 GB per launch).
     constexpr bool STREAMS = NF == 1 || NH == 3;  // the forms that come near the memory system's limit
     constexpr int PX = (NF == 1 && NH == 2) ? kStream : kCached;
     constexpr int PY = kCached;
-    constexpr int PZ = STREAMS ? kStream : kCached;
+    constexpr int PZ = (NF == 1 || (NH == 3 && !REVERSE)) ? kStream : kCached;
     constexpr int PO = STREAMS ? kStream : kCached;
     extern __shared__ __align__(16) unsigned char smem[];
     // LDS map in bytes: [3][x 64*XS | y 64*XS] tiles, [NZ][64*ZS] z tiles, [2][64*PS] P tiles.
