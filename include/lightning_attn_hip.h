@@ -184,7 +184,8 @@ int la_fwd_silu(const void *q, const void *k, const void *v, const float *s, voi
  * one chunk of each sequence at each of them.  It then needs neither warm-up blocks nor collect and scan
  * launches to run as several workgroups per sequence, which is what lets it use 128-column workgroups
  * when b*h alone gives the chip one or two workgroups per compute unit (b*h of 65 .. 128 on 256 CUs,
- * 64 < d <= 128, e <= 128, bf16 / fp16).  The reference recomputes that state in its backward pass
+ * 64 < d <= 128, e <= 128, bf16 / fp16) - or, with d and e both in 129 .. 192, workgroups that take all
+ * columns of a sequence.  The reference recomputes that state in its backward pass
  * (lightning_attn/ops/triton/lightning_attn2.py:240-280) and saves the inputs only (:432); keeping a few
  * states as well is a deviation made for speed.  Gradients agree with la_bwd's to rounding (the state is
  * summed in the same order but its operands are rounded to the tensors' dtype in the other role).
