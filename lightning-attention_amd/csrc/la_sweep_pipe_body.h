@@ -23,12 +23,11 @@
 //   - the P tiles: two LDS buffers (one read, one written);
 //   - the output tile of a block, which the state waves write over the z columns they alone read
 //     and which leaves for memory as whole row segments when that z slot is refilled.
-// NH = 3 is a form of its own for feature dims and column counts of 129 .. 192: one workgroup of FOUR wavefronts
-// covers all (up to 192) columns of a sequence, and every wavefront plays both parts - it fetches and publishes
-// a quarter of the tiles, computes its share of the score tile, and owns three 16-column slabs of the state
-// (144 accumulator registers; with one wavefront per SIMD a wavefront has 512 registers).  The x and y tiles
-// are then read from LDS by four wavefronts per 192 columns instead of six (three state waves in each of two
-// 96-column workgroups), and staged and multiplied into a score tile once per sequence instead of twice.
+// NH = 3 (feature dims and column counts of 129 .. 192): a workgroup covers all (up to 192) columns of a sequence,
+// every state wave owning three 16-column slabs = 144 accumulator registers of state.  The x and y tiles are then
+// staged and multiplied into a score tile once per sequence and block instead of twice, and read from LDS by four
+// state waves instead of six (three in each of two 96-column workgroups).  To fit 256 registers the state waves
+// fetch their fragments without look-ahead and keep their decay factors in LDS (LEAN below).
 // With few (batch, head) sequences the walk is cut into chunks, one workgroup each.  A chunk's
 // incoming state comes either from warm-up blocks (the workgroup first walks everything before its
 // chunk with the state update alone) or, given a workspace, from a scan: the same kernel run once in
@@ -84,8 +83,6 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
     // Threads that fetch, publish and write back the tiles: the 256 of the score waves, which have
     // slack; the state waves' serial chain then holds no memory instructions at all.
     constexpr int NL = 256;
-    constexpr bool MERGED = false;
-    constexpr int NT = MERGED ? 256 : 512;   // threads of the workgroup
     constexpr int CPX = DKH / 8;             // 16-byte chunks per row of an x / y chunk tile
     constexpr int XC = 64 * CPX / NL;        // ... per loader thread
     constexpr bool ROWAL = NL % CPX == 0;    // a thread's chunks lie a whole number of rows apart
@@ -100,6 +97,7 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
     // travels one register set behind them.  NF = 2: the z slice travels with the first feature
     // chunk of its block and is published a block ahead.
     constexpr int ZLAG = (NF == 1 && NH == 2) ? 1 : 0;
+    constexpr bool TOGETHER = NF == 2 && NH == 3;  // see the load slot of `iteration`
     // Cache policy of the global accesses.  Every tile is needed once per workgroup, and the only second readers
     // are a sibling workgroup that runs beside this one: the other 64-column slice of the head, which reads the same
     // x and y, and the other sweep of a pair, which reads this sweep's y as its z and the other way round.  So the
@@ -155,7 +153,7 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const bool state_role = MERGED || wave >= 4;
+    const bool state_role = wave >= 4;
     const int w = wave & 3;
     const int lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int64_t n = a.n;
@@ -189,13 +187,11 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
     //   score waves: cf[4 sl + v]  mask * decay of element v of score tile slot sl
     //   state waves: cf[it]        scale of the inter-block term for token i = 16 it + r
     //                cf[4 + 8 ks + u]  scale of token j = 32 ks + 8 g + u in the state update
-    // (four wavefronts: both sets, the score waves' behind the state waves')
-    constexpr int SC = MERGED ? 20 : 0;
-    float cf[20 + SC];
+    float cf[20];
 #pragma unroll
-    for (int i = 0; i < 20 + SC; ++i) cf[i] = 1.f;
+    for (int i = 0; i < 20; ++i) cf[i] = 1.f;
     float lamB = 1.f;
-    if (MERGED || !state_role) {
+    if (!state_role) {
         const int its[3] = {itA, itB, itB}, jts[3] = {jt0, jt1, jt2};
 #pragma unroll
         for (int sl = 0; sl < 3; ++sl)
@@ -203,7 +199,7 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
             for (int v = 0; v < 4; ++v) {
                 const int i = 16 * its[sl] + r, j = 16 * jts[sl] + 4 * g + v;
                 const int diff = REVERSE ? (j - i) : (i - j);
-                cf[SC + 4 * sl + v] = diff >= 0 ? (DECAY ? expf(-rate * (float)diff) : 1.f) : 0.f;
+                cf[4 * sl + v] = diff >= 0 ? (DECAY ? expf(-rate * (float)diff) : 1.f) : 0.f;
             }
     }
     if (state_role && DECAY) {
@@ -481,23 +477,23 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
             {
                 V4 p;
 #pragma unroll
-                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[0][v] * cf[SC + v]);
+                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[0][v] * cf[v]);
                 *reinterpret_cast<V4*>(smem + opaque(pbase + (16 * itA * PS + 16 * jt0) * E)) = p;
             }
             if (itB >= 0) {
                 V4 p;
 #pragma unroll
-                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[1][v] * cf[SC + 4 + v]);
+                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[1][v] * cf[4 + v]);
                 *reinterpret_cast<V4*>(smem + opaque(pbase + (16 * itB * PS + 16 * jt1) * E)) = p;
 #pragma unroll
-                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[2][v] * cf[SC + 8 + v]);
+                for (int v = 0; v < 4; ++v) p[v] = M::cvt(sacc[2][v] * cf[8 + v]);
                 *reinterpret_cast<V4*>(smem + opaque(pbase + (16 * itB * PS + 16 * jt2) * E)) = p;
             }
         }
     };
 
     // zero both P buffers once: tiles on the masked side of the diagonal are never written
-    for (int c = tid; c < 2 * L::PT / 8; c += NT) reinterpret_cast<uint4*>(smem + PBASE)[c] = make_uint4(0, 0, 0, 0);
+    for (int c = tid; c < 2 * L::PT / 8; c += 512) reinterpret_cast<uint4*>(smem + PBASE)[c] = make_uint4(0, 0, 0, 0);
     // state-wave lane offsets: x fragment halves (row r, columns 4g..), transposed reads of y and
     // of this wave's 16 z columns (row 8g + r/4, columns 4 (r%4)..), P fragments (row r, chunk g)
     const unsigned lane_xq = (r * XS + 4 * g) * E;
@@ -538,7 +534,7 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
 
     // One step: feature chunk HF of block `it`; step number s = NF it + HF.  `xr, yr, zr` hold step
     // s+2 on entry and step s+4 on exit.
-    // `role`: 0 the score waves' part of the step, 1 the state waves', 2 both (four wavefronts).
+    // `role`: 0 the score waves' part of the step, 1 the state waves'.
     auto iteration = [&](auto role, auto hf, const int64_t it, u32x4 (&xr)[XC], u32x4 (&yr)[XC], u32x4 (&zr)[ZC]) __attribute__((always_inline)) {
         constexpr int ROLE = decltype(role)::value;
         constexpr int HF = decltype(hf)::value;
@@ -547,19 +543,28 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
         const int bcur = (int)((unsigned)(it * NF + HF) % 3u);
         const int bnext = bcur == 2 ? 0 : bcur + 1;
         const int bstage = bnext == 2 ? 0 : bnext + 1;
-        if constexpr (ROLE != 1) {
+        if constexpr (ROLE == 0) {
             // publish step s+2 (its buffer was last read in step s-1; the z slot that goes with it
             // still holds an output tile) and refill the registers with step s+4
             constexpr int HS = (HF + 2) % NF, HL = (HF + 4) % NF, HC = (HF + 1) % NF;
             const int64_t bs = it + (HF + 2) / NF;  // block of the step being published
             const int zslot = NZ == 3 ? bstage : (int)((bs - ZLAG) & 1);
             stage_step(std::integral_constant<int, HS>{}, bstage, zslot, xr, yr, zr, it - 1, it > it_first);
-            load_step(std::integral_constant<int, HL>{}, it + (HF + 4) / NF, xr, yr, zr);
+            if constexpr (TOGETHER) {
+                // both halves of a block's rows are asked for in one go, after the second half of the block before has
+                // been published: the 128-byte line in the middle of a 384-byte row is then fetched once
+                if constexpr (HF == NF - 1) {
+                    load_step(std::integral_constant<int, 0>{}, it + 2, xrA, yrA, zrA);
+                    load_step(std::integral_constant<int, 1>{}, it + 2, xrB, yrB, zrB);
+                }
+            } else {
+                load_step(std::integral_constant<int, HL>{}, it + (HF + 4) / NF, xr, yr, zr);
+            }
             // the score tile runs one step ahead of the state waves
             const int64_t bc = it + (HF + 1) / NF;
             if (bc < it_end && bc >= it_first) score_step(std::integral_constant<int, HC>{}, bnext, (int)(bc & 1));
         }
-        if (ROLE != 0 && cols_active) {
+        if (ROLE == 1 && cols_active) {
             const unsigned xq = opaque(bcur * XYB + lane_xq);
             const unsigned yq = opaque(bcur * XYB + YOFF + lane_yt);
             const int zcur = NZ == 3 ? bcur : (int)(it & 1);  // z / out slot of this block
@@ -870,13 +875,7 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
                 for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<f32x4*>(dst + (size_t)(h * KT + kt) * 256) = st[h][kt];
         }
     };
-    if constexpr (MERGED) {
-        prologue();
-        init_state();
-        walk(std::integral_constant<int, 2>{});
-        flush_last();
-        leave_state();
-    } else if (!state_role) {
+    if (!state_role) {
         prologue();
         walk(std::integral_constant<int, 0>{});
         flush_last();
