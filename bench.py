@@ -10,8 +10,9 @@ HBM before the timed region.  Prints ONE JSON line.  ``value`` is the algorithmi
 MFMA rate of the step (flop count of a 64-token block recurrence, 344064 flop per
 token and head, divided by the measured time); ``ms_per_step`` is the same
 measurement in milliseconds: W untimed warm-up steps, then exactly K steps between two
-device synchronisations on the host clock.  The same K steps are also bracketed one by
-one with HIP events (``step_event_ms``: median, min, mean).  ``roofline.traffic`` comes from a committed
+device synchronisations on the host clock.  K more steps right after them are bracketed one by
+one with HIP events (``step_event_ms``: median, min, mean; an event record between two steps costs
+~6 us of idle time, so it is kept out of the timed region).  ``roofline.traffic`` comes from a committed
 rocprofv3 counter summary and is withheld when the kernel sources have changed since it was taken;
 ``parity.literal_fail_frac`` states how often the step's own results miss the tolerance as literally named.
 
@@ -120,20 +121,26 @@ def stats(ts):
 
 def timed_steps(step, warmup, steps):
     """The protocol of the headline figure: `warmup` untimed steps, a synchronisation, exactly
-    `steps` steps on the host clock, a synchronisation; every step also sits between two events."""
+    `steps` steps on the host clock, a synchronisation.  Then the same `steps` steps once more, each
+    between two HIP events, for the per-step statistics: an event record between two steps keeps the
+    next launch from following the last one directly (a gap of ~6 us per step in the kernel trace), so
+    the events stay out of the timed region."""
     import torch
 
     for _ in range(warmup):
         step()
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     ev[0].record()
     for i in range(steps):
         step()
         ev[i + 1].record()
     torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / steps
     return ms, [ev[i].elapsed_time(ev[i + 1]) for i in range(steps)]
 
 
