@@ -531,6 +531,16 @@ def main():
                      "not part of the step: dQ = sweep(dO,V,K) recomputing its state (la_bwd's dQ launch without saved states)",
                      dq_ts, fb, ff, "forward"),
     ]
+    # the step's three launches together: their algorithmic bytes over their launch times
+    step_launch_ms = statistics.median(fwd_save_ts) + statistics.median(bwd_saved_ts)
+    step_launch_bytes = 2 * fb + pair_bytes
+    launches_together = {"bound": "hbm", "achieved": round(step_launch_bytes / (step_launch_ms * 1e-3) / 1e9, 1),
+                         "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": round(step_launch_bytes / (step_launch_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                         "algorithmic_bytes": step_launch_bytes, "launch_ms": round(step_launch_ms, 4),
+                         "note": "forward + dQ + (dK + dV) launches: per-launch algorithmic bytes (dO, k, v are read by "
+                                 "two launches) over la_fwd_save + la_bwd_saved; `roofline` is the forward launch, the "
+                                 "one furthest below the roof"}
     direct_ms = {"la_fwd_save": stats(fwd_save_ts), "la_bwd_saved": stats(bwd_saved_ts),
                  "la_fwd": stats(fwd_ts), "la_bwd": stats(bwd_ts)}
     buf = saved = None
@@ -561,6 +571,7 @@ def main():
         "step_hbm_frac": round(bytes_step / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
         "roofline": roofline,
         "roofline_other_launches": other_launches,
+        "roofline_step_launches": launches_together,
         "entry_points_ms": direct_ms,
     }
     line.update(out)
