@@ -2,14 +2,14 @@
 // barrier per step, for feature dims up to 256.  Included by la_sweep_pipe.hip (feature dim <= 128) and
 // la_sweep_pipe_split.hip (129 .. 256), which instantiate it.
 //
-// One workgroup of 8 wavefronts per (batch, head, 64- or 128-column slice of z/out), 64-token blocks
+// One workgroup of 8 wavefronts per (batch, head, slice of 64, 128 or up to 192 columns of z/out), 64-token blocks
 // walked in order, fp32 state in MFMA accumulators.  The two kinds of wavefronts work on different
 // data at the same time:
 //   waves 0-3 ("score" waves)  do all the memory traffic (two register sets of prefetch, the tiles
 //                              published in LDS two steps ahead, the output tile of the block before
 //                              written back) and compute the masked, decayed score tile P one step
 //                              ahead of the state waves;
-//   waves 4-7 ("state" waves)  own one or two dk x 16 column slabs of the state and finish the
+//   waves 4-7 ("state" waves)  own one, two or three dk x 16 column slabs of the state and finish the
 //                              block: out^T = Lout * (state^T x^T) + z^T P^T, left in LDS, then
 //                              state = lam^64 state + y^T (z * Lupd).
 // A step is a block (NF = 1, feature dim <= 128) or one of the NF = 2 halves of the feature dim of a
@@ -46,7 +46,7 @@
 namespace la {
 
 // DKP: feature dim as padded; NF: halves it is processed in; NH: 16-column accumulator slabs per state
-// wave (a workgroup covers 64 NH columns of z / out).
+// wave (a workgroup covers 64 NH columns of z / out; NH = 3 with DKP = 192 only).
 template <int DKP, int NF, int NH>
 struct PipeLds {
     static_assert(NF == 1 || NF == 2, "one or two feature chunks");
@@ -106,13 +106,14 @@ __device__ __forceinline__ void sweep_pipe_body(const SweepPair& pair, const uns
     // step after its x / y tiles), so the sibling's streamed z read finds it in L2 - and with all four streamed
     // every launch measured slower than with none.  Measured at b4 h32 n8192 d128, ms: la_fwd (64 columns) 0.2253 all
     // cached, 0.2207 as here, 0.2153 with x streamed as well - at 1.137 instead of 1.077 GB of HBM traffic, the
-    // sibling slice's read of x then missing L2 now and then: not taken; dQ in 128-column workgroups 0.2078 -> 0.178;
-    // dK + dV 0.315 -> 0.310 at 1.643 instead of 1.726 GB.  (A kernel that only streams this access pattern: 5.3 TB/s
+    // sibling slice's read of x then missing L2 now and then: not taken; dQ in 128-column workgroups 0.2078 -> 0.190;
+    // dK + dV 0.315 -> 0.302 at 1.616 instead of 1.63 - 1.75 GB.  (A kernel that only streams this access pattern: 5.3 TB/s
     // with cached, 5.9 TB/s with streamed accesses.)  At feature dims above 128 the launches in 64- and 96- / 128-column
     // workgroups are bound by LDS work and the policy made no difference: left cached.  With all columns in one
     // workgroup (NH = 3) they come near the memory side's limit for tiles fetched in half rows (4.6 - 4.8 TB/s for
     // a kernel that only streams that pattern): there the output is streamed, x and y stay cached (the 128-byte
-    // line in the middle of a 384-byte row belongs to both halves and is asked for twice, half a block apart), and
+    // line in the middle of a 384-byte row belongs to both halves; with TOGETHER they are asked for in one load
+    // slot, and streamed they still lost: la_bwd_saved 0.881 against 0.872 ms at b4 h32 n8192 d192), and
     // z is streamed only when walking forward - walking backward the launch is a dK + dV pair, whose z reads are
     // the sibling sweep's y reads of the same moment (b4 h32 n8192 d192: 2.42 instead of 2.74 GB per launch).
     constexpr bool STREAMS = NF == 1 || NH == 3;  // the forms that come near the memory system's limit
