@@ -440,6 +440,32 @@ def test_full_size_against_block_recurrence_on_head_subset(n):
         check(got, (want_o,) + tuple(want_g), torch.bfloat16, "n=%d head (%d,%d)" % (n, bi, hi))
 
 
+@pytest.mark.parametrize("b, n, d", [(4, 8192, 192), (8, 4096, 192), (4, 4096, 160)])
+def test_full_size_at_feature_dims_129_to_192(b, n, d):
+    """h = 32 at d = e = 192 / 160 with 128 and 256 sequences, the shapes the all-column workgroups are planned
+    for (dK + dV, dQ from the forward pass's states; from 256 sequences on the forward launch as well): three
+    (batch, head) pairs against the fp64 block-recurrence oracle, and the whole result against the run with
+    64-column workgroups throughout and no saved states (o, dk, dv bit for bit; dq to rounding where states
+    were used)."""
+    h = 32
+    q, k, v, do = _full_inputs(b, h, n, d)
+    s = _build_slope_tensor(h)
+    got = run_hip(q, k, v, s, do)
+    for bi, hi in ((0, 0), (1, 13), (b - 1, 31)):
+        sub = [t[bi:bi + 1, hi:hi + 1].float().cpu() for t in (q, k, v, do)]
+        ss = s[hi:hi + 1]
+        want_o = oracle.block_recurrence_fwd(sub[0], sub[1], sub[2], ss, 64)
+        want_g = oracle.block_recurrence_bwd(sub[0], sub[1], sub[2], ss, sub[3], 64)
+        check([t[bi:bi + 1, hi:hi + 1] for t in got], (want_o,) + tuple(want_g), torch.bfloat16,
+              "d=%d b=%d n=%d head (%d,%d)" % (d, b, n, bi, hi))
+    narrow = run_hip(q, k, v, s, do, wide=False, save_states=False)
+    for name, a, c in zip(("o", "dq", "dk", "dv"), got, narrow):
+        if name == "dq":
+            assert rel_norm(a, c.float()) < 3e-3, name
+        else:
+            assert torch.equal(a, c), name
+
+
 def test_very_long_sequence_few_heads():
     """n = 262144 (4096 blocks), b1 h2: the chunked walk at its longest; the slow-decay head against the
     fp64 block recurrence, and no decay (a state that keeps growing) as well."""
