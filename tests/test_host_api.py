@@ -120,6 +120,47 @@ def test_workspace_query_is_consistent():
     assert L.la_workspace_bytes_opts(0, 1, 8, 65536, 128, 128, 0, ctypes.byref(bad)) == 0
 
 
+def test_saved_state_query_is_consistent():
+    """Properties of la_saved_state_bytes / la_saved_state_interval over a grid of shapes (host logic only; 256 CUs
+    assumed without a device): a whole number m of d x e float matrices per sequence, boundaries a multiple of 64
+    tokens apart and all inside the sequence, m + 1 chunks that give every CU at most one workgroup; nothing for
+    float32, for feature dims the pair has no kernel forms for, for shapes whose sequences fill the chip or leave it
+    to the chunked plans, and nothing when the launch options pin another form."""
+    L = _lib.lib()
+    used = set()
+    for b, h in ((1, 8), (2, 12), (1, 64), (3, 24), (4, 20), (4, 32), (5, 32), (8, 32)):
+        for n in (64, 512, 1000, 4096, 8192, 65536):
+            for d, e in ((64, 64), (72, 128), (128, 128), (128, 96), (96, 160), (136, 136), (192, 192), (176, 144), (192, 128), (256, 256)):
+                for dtype in (0, 1, 2):
+                    if dtype == 2 and (d > 128 or e > 128):
+                        continue
+                    nbytes = L.la_saved_state_bytes(b, h, n, d, e, dtype, None)
+                    step = L.la_saved_state_interval(b, h, n, d, e, dtype, None)
+                    assert (nbytes == 0) == (step == 0)
+                    small = 64 < d <= 128 and e <= 128
+                    big = 128 < d <= 192 and 128 < e <= 192
+                    units8 = (b * h + 7) // 8 * 8
+                    if big and units8 * 3 <= 256:  # the forward pass then runs in 64-column workgroups: no form that saves
+                        big = False
+                    if dtype == 2 or not (small or big) or not 64 < b * h <= 128 or n < 512:
+                        assert nbytes == 0, (b, h, n, d, e, dtype)
+                        continue
+                    assert nbytes > 0, (b, h, n, d, e, dtype)
+                    m, rest = divmod(nbytes, b * h * d * e * 4)
+                    assert rest == 0 and m >= 1 and step % 64 == 0
+                    assert m * step < n <= (m + 1) * step + 63
+                    assert (b * h + 7) // 8 * 8 * (m + 1) <= 256
+                    used.add((small, big))
+                    for kw in (dict(chunks=2), dict(wide=_lib.LA_OPT_ON), dict(wide=_lib.LA_OPT_ALL), dict(scan=_lib.LA_OPT_ON)):
+                        o = _lib.LaunchOpts(kw.get("chunks", 0), kw.get("scan", 0), kw.get("wide", 0), 0, 0)
+                        assert L.la_saved_state_bytes(b, h, n, d, e, dtype, ctypes.byref(o)) == 0
+    assert used == {(True, False), (False, True)}
+    # the headline shape: one matrix of 128 x 128 floats per sequence, at the middle of the sequence
+    assert L.la_saved_state_bytes(4, 32, 8192, 128, 128, 0, None) == 128 * 128 * 128 * 4
+    assert L.la_saved_state_interval(4, 32, 8192, 128, 128, 0, None) == 4096
+    assert L.la_saved_state_bytes(4, 32, 8192, 192, 192, 0, None) == 128 * 192 * 192 * 4
+
+
 def test_static_scratch_holds_every_plan_of_the_forward():
     """la_fwd_static rejects shapes whose plan needs more than its static array (LA_E_WORKSPACE): over a
     grid of shapes, on a chip of 256 compute units (what the library plans for without a device), no
