@@ -466,6 +466,16 @@ def test_full_size_at_feature_dims_129_to_192(b, n, d):
             assert torch.equal(a, c), name
 
 
+@pytest.mark.parametrize("b, h, n, d, e", [(2, 4, 300, 128, 128), (1, 3, 200, 256, 256), (2, 2, 260, 192, 128), (1, 2, 130, 64, 160)])
+def test_all_columns_option_is_the_librarys_choice_where_it_has_no_form(b, h, n, d, e):
+    """wide="all" (LA_OPT_ALL) names a form that exists for d and e both in 129 .. 192; elsewhere the option is
+    accepted and means the library's own choice: same bits as without it."""
+    q, k, v, do = make_inputs(b, h, n, d, e, torch.bfloat16, 0.6, seed=n + d)
+    s = _build_slope_tensor(h)
+    for a, c in zip(run_hip(q, k, v, s, do, wide="all"), run_hip(q, k, v, s, do)):
+        assert torch.equal(a, c)
+
+
 def test_very_long_sequence_few_heads():
     """n = 262144 (4096 blocks), b1 h2: the chunked walk at its longest; the slow-decay head against the
     fp64 block recurrence, and no decay (a state that keeps growing) as well."""
