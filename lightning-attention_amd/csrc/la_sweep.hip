@@ -271,6 +271,10 @@ SavedPlan plan_saved(int64_t bh, int64_t n, int64_t d, int64_t e, int dtype, con
     if (!big && (d <= 64 || d > 128 || e > 128)) return none;
     if (opts.chunks != 0 || opts.wide == LA_OPT_ON || opts.wide == LA_OPT_ALL || opts.scan == LA_OPT_ON) return none;
     const int64_t nblk = (n + 63) / 64, cus = num_cus(), units8 = (bh + 7) / 8 * 8;
+    // Short sequences: writing the states and starting from them costs what the wider workgroups save
+    // (b4 h32 d128 fwd+bwd, with / without: n = 512 0.060 / 0.056 ms, 1024 0.097 / 0.096, 2048 0.176 / 0.181, 4096
+    // 0.341 / 0.357; d = 192: n = 1024 0.160 / 0.158, 2048 0.319 / 0.332).
+    if (nblk < 24) return none;
     const int fwd_width = big ? 1 : 0, dq_width = big ? 2 : 1;
     // the forward pass as planned: that width, one walk per sequence
     if (column_width(bh, n, d, e, 1, (size_t)-1, opts) != fwd_width) return none;
