@@ -228,7 +228,7 @@ int la_bwd_saved(const void *q, const void *k, const void *v, const float *s, co
  * No counterpart in the reference (its operators allocate through torch,
  * lightning_attn/ops/triton/lightning_attn2.py:408).
  */
-#define LA_STATIC_SCRATCH_BYTES (16u << 20)
+#define LA_STATIC_SCRATCH_BYTES (48u << 20)
 int la_fwd_static(const void *q, const void *k, const void *v, const float *s, void *o,
                   int64_t b, int64_t h, int64_t n, int64_t d, int64_t e, int dtype, void *stream);
 

@@ -89,7 +89,7 @@ struct ScanPlan {
 // plus two more launches and the scan (16 us measured, and 10 for the host's share).
 // `width` of a workgroup: 0 = 64 columns of z / out, 1 = 128 (96 where there are 192 to share out), 2 = all
 // (129 .. 192) columns in a workgroup of four wavefronts.
-static const double kWholeBlockUs = 4.2;
+static const double kWholeBlockUs = 3.9;
 static double block_us(int64_t dk, int width) {
     if (dk <= 64) return 1.0;
     if (dk <= 128) return width ? 1.75 : 1.4;
@@ -170,21 +170,27 @@ static bool wide_columns(int64_t bh, int64_t n, int64_t dk, int64_t dv, int npro
     return (wide + cus - 1) / cus * 5 < (narrow + cus - 1) / cus * 4;
 }
 
-// Feature dims and columns of 129 .. 192: one workgroup of four wavefronts can take all columns of a sequence
-// (la_sweep_pipe_body.h, NH = 3).  It does per block what two 96-column workgroups do in kWholeBlockUs against
-// 3.0 us each, so it is the form wherever the 64-column one does not already give every workgroup a CU of its own:
-// with that few sequences the narrow workgroups and their chunks spread better over the chip.
+// Estimated duration (us) of one launch of nprod sweeps in workgroups of width code `width`, by the figures
+// above: rounds of workgroups where they fill the chip, else the better of the two chunk plans.
+static double width_us(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int width, size_t scratch, const Opts& opts) {
+    const int64_t cus = num_cus(), nblk = (n + 63) / 64, wgs = (bh + 7) / 8 * 8 * slices(dk, dv, width) * nprod;
+    if (wgs * 2 > cus) return (double)((wgs + cus - 1) / cus) * (double)nblk * block_us(dk, width);
+    const ScanPlan pl = plan_scan(bh, n, dk, dv, nprod, width, opts);
+    return pl.nchunk > 1 && pl.bytes <= scratch ? pl.us : warm_up_us(bh, n, dk, dv, nprod, width);
+}
+
+// Feature dims and columns of 129 .. 192: one workgroup can take all columns of a sequence (la_sweep_pipe_body.h,
+// NH = 3), at kWholeBlockUs per block against 3.0 us for each of two 96-column workgroups or 2.1 us for each of
+// three 64-column ones.  Taken where it is estimated at least 3 % faster than the choice among the narrower forms:
+// fewer rounds of workgroups with many sequences (b*h = 160 at n = 4096: la_fwd 0.241 against 0.300 ms, la_bwd 0.703
+// against 0.878), shorter chunks with few (b*h = 24 at n = 16384: la_fwd 0.185 against 0.309 ms; b*h = 48 at n = 4096:
+// 0.104 / 0.272 against 0.141 / 0.317).
 // Returns the width code of the launch: 0 / 1 as wide_columns has it, or 2.  opts.wide overrides the choice.
 static int column_width(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, size_t scratch, const Opts& opts) {
     const int wide = wide_columns(bh, n, dk, dv, nprod, scratch, opts) ? 1 : 0;
     if (dk <= 128 || dk > 192 || dv <= 128 || dv > 192) return wide;
     if (opts.wide != LA_OPT_AUTO) return opts.wide == LA_OPT_ALL ? 2 : wide;
-    const int64_t cus = num_cus(), nblk = (n + 63) / 64, units = (bh + 7) / 8 * 8 * nprod;
-    if (units * slices(dk, dv, 0) <= cus) return wide;
-    auto rounds = [&](int64_t wgs) { return (double)((wgs + cus - 1) / cus); };
-    const double now = rounds(units * slices(dk, dv, wide)) * block_us(dk, wide);
-    const double whole = (units * 2 <= cus ? warm_up_frac(units, nblk) : rounds(units)) * block_us(dk, 2);
-    return whole < now ? 2 : wide;
+    return width_us(bh, n, dk, dv, nprod, 2, scratch, opts) < 0.97 * width_us(bh, n, dk, dv, nprod, wide, scratch, opts) ? 2 : wide;
 }
 
 // The column slices of a sweep whose workgroups have width code `width` (make_args leaves 64-column slices).

@@ -169,7 +169,7 @@ def test_static_scratch_holds_every_plan_of_the_forward():
     text = open(HEADER).read()
     cap = re.search(r"#define LA_STATIC_SCRATCH_BYTES \((\d+)u << (\d+)\)", text)
     cap = int(cap.group(1)) << int(cap.group(2))
-    assert cap == 16 << 20
+    assert cap == 48 << 20
     worst = 0
     for b, h in ((1, 1), (1, 2), (1, 3), (1, 4), (1, 8), (2, 12), (1, 16), (1, 32), (3, 5), (1, 64), (1, 120)):
         for n in (1000, 4096, 8192, 65536, 1 << 20):

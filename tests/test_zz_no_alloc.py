@@ -53,7 +53,7 @@ def test_static_scratch_forward_matches_workspace_forward():
     results = []
     for i, (b, h, n, d, e) in enumerate(shapes):
         need = L.la_workspace_bytes(0, b, h, n, d, e, 0)
-        assert 0 < need <= 16 << 20, (b, h, n, d, e, need)
+        assert 0 < need <= 48 << 20, (b, h, n, d, e, need)
         q, k, v = _inputs(b, h, n, d, e, 100 + i)
         s = _build_slope_tensor(h).to(DEV).float().contiguous() if i != 1 else None
         print("la_fwd_static case", (b, h, n, d, e), "workspace bytes", need, flush=True)
