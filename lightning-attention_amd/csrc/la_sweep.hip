@@ -134,6 +134,15 @@ static ScanPlan plan_scan(int64_t bh, int64_t n, int64_t dk, int64_t dv, int npr
     return pl;
 }
 
+// Estimated duration (us) of one launch of nprod sweeps in workgroups of width code `width`, by the figures
+// above: rounds of workgroups where they fill the chip, else the better of the two chunk plans.
+static double width_us(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int width, size_t scratch, const Opts& opts) {
+    const int64_t cus = num_cus(), nblk = (n + 63) / 64, wgs = (bh + 7) / 8 * 8 * slices(dk, dv, width) * nprod;
+    if (wgs * 2 > cus) return (double)((wgs + cus - 1) / cus) * (double)nblk * block_us(dk, width);
+    const ScanPlan pl = plan_scan(bh, n, dk, dv, nprod, width, opts);
+    return pl.nchunk > 1 && pl.bytes <= scratch ? pl.us : warm_up_us(bh, n, dk, dv, nprod, width);
+}
+
 // The pipelined kernel can give each workgroup 128 columns of z / out instead of 64: the score tile
 // and the x / y tiles are then produced once per 128 output columns, and the power-limited kernel
 // turns the saved work into time (dK + dV at the headline shape: 0.31 against 0.415 ms) - as long
@@ -146,13 +155,15 @@ static bool wide_columns(int64_t bh, int64_t n, int64_t dk, int64_t dv, int npro
     if (dk > 128) {
         // Feature dims 129 .. 256: 128-column workgroups where that makes fewer slices.
         // They pay when the 64-column form needs more rounds of workgroups than the chip has CUs for
-        // (a wide workgroup takes about 1.4 times as long); with few sequences the 64-column form has
-        // more workgroups to spread over the CUs and stays.
+        // (a wide workgroup takes about 1.4 times as long), and with few sequences on a long walk, where half as
+        // many workgroups mean twice the chunks (d = e = 256 fwd+bwd: b1 h8 n16384 0.42 against 0.58 ms, b2 h12 n16384
+        // 1.16 against 1.59, b2 h12 n4096 0.33 against 0.41); in between the 64-column form has more workgroups to
+        // spread over the CUs and stays.
         const int64_t ws = wide_slices(dv), ns = (dv + 63) / 64;
         if (ws >= ns) return false;
         if (opts.wide != LA_OPT_AUTO) return opts.wide == LA_OPT_ON;
         const int64_t cus = num_cus(), units = (bh + 7) / 8 * 8 * nprod, wide = units * ws, narrow = units * ns;
-        if (narrow <= cus) return false;
+        if (narrow <= cus) return width_us(bh, n, dk, dv, nprod, 1, scratch, opts) < 0.9 * width_us(bh, n, dk, dv, nprod, 0, scratch, opts);
         return (wide + cus - 1) / cus * 7 < (narrow + cus - 1) / cus * 5;
     }
     if (dv <= 64 || dv > 128) return false;
@@ -163,20 +174,13 @@ static bool wide_columns(int64_t bh, int64_t n, int64_t dk, int64_t dv, int npro
         // Every 64-column workgroup gets a CU of its own.  With so few of them that a long walk is cut
         // into chunks from scanned states, rather half as many workgroups of 128 columns and twice the chunks
         // (b1 h32 n8192 fwd+bwd 0.28 against 0.34 ms, b1 h4 n65536 0.46 against 0.62).
-        if (narrow * 2 > cus) return false;
+        // (in between: one 128-column workgroup per sequence only where the second 64-column slice would be half
+        // empty - d = e = 96, b*h = 96: la_fwd 0.321 against 0.359 ms at n = 16384, la_bwd 0.78 against 0.82)
+        if (narrow * 2 > cus) return dv <= 96;
         const ScanPlan w = plan_scan(bh, n, dk, dv, nprod, true, opts), nw = plan_scan(bh, n, dk, dv, nprod, false, opts);
         return w.nchunk > 1 && w.bytes <= scratch && w.us < (nw.bytes <= scratch ? nw.us : warm_up_us(bh, n, dk, dv, nprod, false));
     }
     return (wide + cus - 1) / cus * 5 < (narrow + cus - 1) / cus * 4;
-}
-
-// Estimated duration (us) of one launch of nprod sweeps in workgroups of width code `width`, by the figures
-// above: rounds of workgroups where they fill the chip, else the better of the two chunk plans.
-static double width_us(int64_t bh, int64_t n, int64_t dk, int64_t dv, int nprod, int width, size_t scratch, const Opts& opts) {
-    const int64_t cus = num_cus(), nblk = (n + 63) / 64, wgs = (bh + 7) / 8 * 8 * slices(dk, dv, width) * nprod;
-    if (wgs * 2 > cus) return (double)((wgs + cus - 1) / cus) * (double)nblk * block_us(dk, width);
-    const ScanPlan pl = plan_scan(bh, n, dk, dv, nprod, width, opts);
-    return pl.nchunk > 1 && pl.bytes <= scratch ? pl.us : warm_up_us(bh, n, dk, dv, nprod, width);
 }
 
 // Feature dims and columns of 129 .. 192: one workgroup can take all columns of a sequence (la_sweep_pipe_body.h,

@@ -74,10 +74,10 @@ CASES = [
     # b, h, n, d, e, dtype, decay, token_major
     (4, 32, 1536, 128, 128, torch.bfloat16, True, False),   # the benchmark's b*h: 2 chunks
     (3, 24, 1700, 128, 128, torch.bfloat16, True, False),   # 72 sequences: 3 chunks, the last one short and ragged
-    (4, 32, 1555, 128, 96, torch.float16, True, False),     # e < d, fp16, ragged
+    (4, 32, 1555, 128, 104, torch.float16, True, False),    # e < d, fp16, ragged
     (2, 64, 1900, 72, 128, torch.bfloat16, False, False),   # no decay, d off the 64 grid
     (4, 32, 2048, 128, 128, torch.bfloat16, True, True),    # projection layout, used in place
-    (4, 25, 1664, 96, 80, torch.bfloat16, True, True),
+    (4, 25, 1664, 96, 112, torch.bfloat16, True, True),
     # feature dims 129 .. 192: the forward pass in two column slices, dQ with all its columns in one workgroup
     (4, 32, 1536, 192, 192, torch.bfloat16, True, False),
     (4, 30, 1700, 176, 144, torch.float16, True, True),     # ragged, d != e, projection layout
@@ -171,7 +171,8 @@ def test_saved_states_through_autograd_and_the_opt_out():
 @pytest.mark.parametrize("b, h, n, d, e, dtype", [(1, 8, 4096, 128, 128, torch.bfloat16), (8, 32, 512, 128, 128, torch.bfloat16),
                                                  (4, 32, 1024, 64, 64, torch.bfloat16), (4, 32, 1024, 256, 256, torch.bfloat16),
                                                  (4, 32, 1024, 192, 128, torch.bfloat16),
-                                                 (4, 32, 128, 128, 128, torch.bfloat16), (4, 32, 1024, 128, 128, torch.bfloat16)])
+                                                 (4, 32, 128, 128, 128, torch.bfloat16), (4, 32, 1024, 128, 128, torch.bfloat16),
+                                                 (4, 32, 2048, 128, 96, torch.bfloat16)])
 def test_shapes_without_saved_states_are_the_plain_entry_points(b, h, n, d, e, dtype):
     L = _lib.lib()
     assert L.la_saved_state_bytes(b, h, n, d, e, CODE[dtype], None) == 0
