@@ -381,17 +381,19 @@ int sweep_bwd_once(const SweepIO& dq, const SweepIO& dk, const SweepIO& dv, cons
     const int64_t cus = num_cus(), nblk = (n + 63) / 64, nslice = (d + 63) / 64;
     const int64_t wgs = (bh + 7) / 8 * 8 * nslice * 3;  // one chunk each
     if (forced == 0) {
-        if (wgs > cus) return LA_E_UNSUPPORTED;
+        // (up to two rounds of workgroups: on a short walk one launch of twice as many 64-column workgroups as
+        // there are CUs still beats two launches - b1 h48 n2048 d192: la_bwd 0.138 against 0.162 ms)
+        if (wgs > 2 * cus) return LA_E_UNSUPPORTED;
         // what the separate launches would take, by the estimates behind their own plans
         const bool ws_ok = ws && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0;
         double separate = 0.0;
         for (int nprod = 1; nprod <= 2; ++nprod) {
-            const int wide = column_width(bh, n, d, d, nprod, ws_ok ? ws_bytes : 0, opts);
-            const ScanPlan pl = plan_scan(bh, n, d, d, nprod, wide, opts);
-            separate += pl.nchunk > 1 && ws_ok && ws_bytes >= pl.bytes ? pl.us : warm_up_us(bh, n, d, d, nprod, wide);
+            const size_t scratch = ws_ok ? ws_bytes : 0;
+            separate += width_us(bh, n, d, d, nprod, column_width(bh, n, d, d, nprod, scratch, opts), scratch, opts);
         }
-        // here: the longest workgroup of 3 * wgs/3 * c warm-up chunked ones
-        if (warm_up_frac(wgs, nblk) * (double)nblk * block_us(d, false) >= separate) return LA_E_UNSUPPORTED;
+        // here: the longest workgroup of 3 * wgs/3 * c warm-up chunked ones, or two rounds of single walks
+        const double rounds = wgs > cus ? 2.0 : 1.0;
+        if (rounds * warm_up_frac(wgs, nblk) * (double)nblk * block_us(d, false) >= separate) return LA_E_UNSUPPORTED;
     }
     SweepBoth b;
     b.fwd.nprod = 1;
