@@ -419,8 +419,8 @@ int sweep_bwd_once(const SweepIO& dq, const SweepIO& dk, const SweepIO& dv, cons
 }
 
 // The same for two sweeps of one shape and opposite directions (dQ and dK of a backward pass with
-// d != e: both contract over e and produce d columns): one launch where they fit on the chip together
-// and separate launches are not estimated faster; LA_E_UNSUPPORTED otherwise.
+// d != e: both contract over e and produce d columns): one launch where separate launches are not estimated
+// faster (they fit on the chip together, or share rounds of workgroups); LA_E_UNSUPPORTED otherwise.
 int sweep_fwd_rev_once(const SweepIO& fwd, const SweepIO& rev, const float* s, int64_t bh, int64_t h, int64_t n, int64_t dk,
                        int64_t dv, int dtype, void* ws, size_t ws_bytes, const Opts& opts, hipStream_t st) {
     if (dtype != LA_BF16 && dtype != LA_FP16) return LA_E_UNSUPPORTED;
@@ -430,12 +430,16 @@ int sweep_fwd_rev_once(const SweepIO& fwd, const SweepIO& rev, const float* s, i
     const int64_t cus = num_cus(), nblk = (n + 63) / 64, nslice = (dv + 63) / 64;
     const int64_t wgs = (bh + 7) / 8 * 8 * nslice * 2;
     if (forced == 0) {
-        if (wgs > cus) return LA_E_UNSUPPORTED;
+        // (up to three rounds of workgroups: where each sweep alone leaves its last round mostly empty, the two
+        // together need fewer rounds - d192 e128 b*h = 96, 288 workgroups a sweep: la_bwd 0.215 against 0.261 ms at
+        // n = 2048; d256 e128 b*h = 80: 0.229 against 0.274)
+        if (wgs > 3 * cus) return LA_E_UNSUPPORTED;
         const bool ws_ok = ws && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0;
-        const int wide = column_width(bh, n, dk, dv, 1, ws_ok ? ws_bytes : 0, opts);
-        const ScanPlan pl = plan_scan(bh, n, dk, dv, 1, wide, opts);
-        const double separate = 2.0 * (pl.nchunk > 1 && ws_ok && ws_bytes >= pl.bytes ? pl.us : warm_up_us(bh, n, dk, dv, 1, wide));
-        if (warm_up_frac(wgs, nblk) * (double)nblk * block_us(dk, false) >= separate) return LA_E_UNSUPPORTED;
+        const size_t scratch = ws_ok ? ws_bytes : 0;
+        const double separate = 2.0 * width_us(bh, n, dk, dv, 1, column_width(bh, n, dk, dv, 1, scratch, opts), scratch, opts);
+        const int64_t rounds = (wgs + cus - 1) / cus;
+        const double share = rounds > 1 ? (double)rounds : warm_up_frac(wgs, nblk);
+        if (share * (double)nblk * block_us(dk, false) >= separate) return LA_E_UNSUPPORTED;
     }
     SweepBoth b;
     b.fwd.nprod = b.rev.nprod = 1;
