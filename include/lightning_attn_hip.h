@@ -92,7 +92,7 @@ typedef struct la_launch_opts {
     int32_t scan;   /* start chunks from scanned states in the workspace: LA_OPT_AUTO (where estimated
                        faster and the workspace suffices) / LA_OPT_OFF (warm-up blocks only)            */
     int32_t wide;   /* output columns per workgroup: AUTO / OFF (64) / ON (128, or two equal slices) /
-                       LA_OPT_ALL (d and e in 129..192: all columns in a workgroup of four wavefronts;
+                       LA_OPT_ALL (d and e in 129..192: all columns of a sequence in one workgroup;
                        as AUTO elsewhere)                                                               */
     int32_t paired; /* backward, d == e: dK and dV in one launch: AUTO (yes) / OFF (one after the other) */
     int32_t once;   /* backward, few sequences: every sweep in one launch: AUTO / OFF / ON               */

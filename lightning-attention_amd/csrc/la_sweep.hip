@@ -88,7 +88,7 @@ struct ScanPlan {
 // workgroup runs the fraction `frac` of a single walk.  Scanned states: a chunk one and a half times,
 // plus two more launches and the scan (16 us measured, and 10 for the host's share).
 // `width` of a workgroup: 0 = 64 columns of z / out, 1 = 128 (96 where there are 192 to share out), 2 = all
-// (129 .. 192) columns in a workgroup of four wavefronts.
+// (129 .. 192) columns of a sequence in one workgroup.
 static const double kWholeBlockUs = 3.9;
 static double block_us(int64_t dk, int width) {
     if (dk <= 64) return 1.0;
