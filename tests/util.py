@@ -23,5 +23,5 @@ def assert_close_scaled(a, ref, rtol=2e-2, atol=2e-2, what=""):
         rms = ref.pow(2).mean().sqrt()
     bound = atol * rms.clamp_min(1.0) + rtol * ref.abs()
     bad = (a - ref).abs() > bound
-    assert not bad.any(), "%s: %d of %d elements outside tolerance (max err %.3e, max rms(ref) %.3e)" % (
-        what, int(bad.sum()), bad.numel(), (a - ref).abs().max().item(), rms.max().item())
+    assert not bad.any(), "%s: %d of %d elements outside tolerance (max err %.3e, max rms(ref) %.3e), the first at %s" % (
+        what, int(bad.sum()), bad.numel(), (a - ref).abs().max().item(), rms.max().item(), bad.nonzero()[:12].tolist())
